@@ -1,0 +1,132 @@
+/*
+ * moe_hip.h -- C ABI of libmoe_hip.so: the MoE expert forward path of
+ * jax-gpt's Qwen3.5 / DeepSeek-V3-style MoE layer as hand-written HIP kernels
+ * for gfx950 (MI355X).
+ *
+ * Every entry point is enqueue-only on the caller's stream: no device
+ * synchronisation, no host read-back, no allocation.  The caller owns every
+ * buffer, including the workspace (size from moe_workspace_bytes).  Inputs are
+ * read-only, outputs are fully overwritten.  Return value 0 = ok, < 0 = one of
+ * MOE_ERR_*; moe_last_error() gives the thread-local message.
+ *
+ * Layouts (all row-major, device pointers, 16-byte aligned):
+ *   logits   (M, E)  f32          router logits
+ *   idx      (M, k)  int32        selected experts, value-descending, ties -> lower index
+ *   w        (M, k)  f32          routing weights
+ *   x        (M, D)  bf16         hidden states
+ *   xq / sx  (R, K) e4m3fn / (R, K/128) f32     activations, 1x128 scale groups
+ *   wq / sw  (E, N, K) e4m3fn / (E, N/128, K/128) f32   weights, K contiguous,
+ *            128x128 scale blocks; real value = code * scale  ("weight_scale_inv")
+ *   flat index f = t*k + s; sorted position p; R = M*k
+ *
+ * Reference citations are to ultrons/jax-gpt, jax_gpt/models/qwen35/.
+ */
+#ifndef MOE_HIP_H
+#define MOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MOE_OK 0
+#define MOE_ERR_BAD_SHAPE (-1)
+#define MOE_ERR_BAD_ALIGN (-2)
+#define MOE_ERR_WORKSPACE_TOO_SMALL (-3)
+#define MOE_ERR_HIP (-4)
+#define MOE_ERR_NULL (-5)
+
+#define MOE_ROUTING_SOFTMAX 0          /* moe.py:37-55 */
+#define MOE_ROUTING_SIGMOID_GROUPED 1  /* DeepSeek-V3 group-limited router (not in the reference) */
+
+typedef void* moe_stream_t; /* a hipStream_t */
+
+int moe_abi_version(void);
+const char* moe_last_error(void);
+
+/* moe.py:51-53 (softmax in f32, lax.top_k, renormalise).  E <= 1024, k <= 32, k <= E. */
+int moe_route_softmax_topk(const float* logits, int M, int E, int k, int renorm,
+                           int32_t* idx, float* w, moe_stream_t stream);
+
+/* DeepSeek-V3 router: sigmoid scores, +bias for selection only, group score = sum of
+ * the group's top-2, keep topk_group groups, top-k among them, weights = un-biased
+ * scores (renormalised with +1e-20) * routed_scale.  Replaces moe.py:37-55 for the
+ * DeepSeek-shaped configs.  bias may be NULL.  E <= 1024, n_group <= 64. */
+int moe_route_sigmoid_grouped(const float* logits, const float* bias, int M, int E, int n_group,
+                              int topk_group, int k, int renorm, float routed_scale,
+                              int32_t* idx, float* w, moe_stream_t stream);
+
+/* moe.py:58-80 (_sort_and_group): stable counting sort of the flat (token, slot)
+ * list by expert id.  Outputs group_sizes (E), group_offsets (E+1), sorted_token_ids
+ * (R), sort_order (R), inv_perm (R); any of the last three may be NULL. */
+size_t moe_permute_workspace_bytes(int M, int k, int E);
+int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* group_sizes,
+                int32_t* group_offsets, int32_t* sorted_token_ids, int32_t* sort_order,
+                int32_t* inv_perm, void* ws, size_t ws_bytes, moe_stream_t stream);
+
+/* 1x128 activation quantiser (replaces fp8.py:30-45's per-row quantiser):
+ * scale = 448/amax, q = e4m3(clamp(x*scale)), sx = 1/scale.  K % 128 == 0. */
+int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream);
+
+/* 128x128 weight block quantiser (replaces quantize.py:18-42's per-row quantiser;
+ * layout (E, out, in) as quantize.py:31-35).  src_is_f32: 0 = bf16 source, 1 = f32. */
+int moe_quant_weight_block(const void* w, int src_is_f32, int E, int N, int K, uint8_t* wq,
+                           float* sw, moe_stream_t stream);
+
+/* moe.py:85-86 + silu*mul of :87, fused: for rows [group_offsets[e], group_offsets[e+1])
+ * h = silu(x . Wgate[e]^T) * (x . Wup[e]^T), then 1x128 fp8 quantisation of h.
+ * row_ids (R) maps sorted position -> row of xq/sx (the gather of moe.py:79 without
+ * materialising x_sorted); NULL = identity (pre-dispatched rows).  D, I % 128 == 0. */
+size_t moe_gemm_workspace_bytes(int R, int E, int N_out);
+int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+                               const uint8_t* w_gate, const float* sw_gate,
+                               const uint8_t* w_up, const float* sw_up,
+                               const int32_t* group_offsets, int E, int R, int D, int I,
+                               uint8_t* hq, float* sh, void* ws, size_t ws_bytes,
+                               moe_stream_t stream);
+
+/* moe.py:87 (the third ragged_dot): y = h . Wdown[e]^T, bf16 out (R, D). */
+int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
+                      const float* sw_down, const int32_t* group_offsets, int E, int R, int I,
+                      int D, void* y_bf16, void* ws, size_t ws_bytes, moe_stream_t stream);
+
+/* moe.py:90-94 (_scatter_back) as a deterministic gather: out[t] = sum_s w[t,s] *
+ * y[inv_perm[t*k+s]] (+ shared[t]) in f32, one bf16 rounding.  shared may be NULL
+ * (moe.py:281 adds the shared expert's output). */
+int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
+                const void* shared_bf16, int M, int k, int D, void* out_bf16, moe_stream_t stream);
+
+/* The whole path (moe.py:97-114 + 225-232 + 281): router logits in, combined hidden
+ * states out. */
+typedef struct MoeForwardArgs {
+  int M, D, E, k, I;       /* tokens, hidden, routed experts, top-k, expert intermediate */
+  int SI;                  /* shared-expert intermediate, 0 = no shared expert */
+  int routing;             /* MOE_ROUTING_* */
+  int n_group, topk_group; /* sigmoid_grouped only */
+  int renorm;
+  float routed_scale;
+  const void* x;           /* (M, D) bf16 */
+  const float* logits;     /* (M, E) */
+  const float* bias;       /* (E) or NULL */
+  const uint8_t *w_gate, *w_up, *w_down;    /* (E,I,D) (E,I,D) (E,D,I) */
+  const float *sw_gate, *sw_up, *sw_down;
+  const uint8_t *ws_gate, *ws_up, *ws_down; /* shared expert (1,SI,D) (1,SI,D) (1,D,SI) or NULL */
+  const float *sws_gate, *sws_up, *sws_down;
+  void* out;               /* (M, D) bf16 */
+  /* optional debug outputs (NULL to skip): the integer results the parity tests check */
+  int32_t* out_idx;        /* (M, k) */
+  float* out_w;            /* (M, k) */
+  int32_t* out_group_sizes;      /* (E) */
+  int32_t* out_sorted_token_ids; /* (R) */
+  int32_t* out_inv_perm;         /* (R) */
+} MoeForwardArgs;
+
+size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI);
+int moe_forward(const MoeForwardArgs* args, void* ws, size_t ws_bytes, moe_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOE_HIP_H */

@@ -1,0 +1,144 @@
+// Error reporting and the whole-path entry point of the C ABI.
+//
+// moe_forward = jax_gpt/models/qwen35/moe.py:97-114 (expert_forward_single) fed by
+// router logits, plus the shared expert of moe.py:225-232 and the add of :281.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "moe_common.h"
+
+static thread_local char g_err[512] = "";
+
+int moe_set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int moe_check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return MOE_OK;
+  return moe_set_error(MOE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+extern "C" int moe_abi_version(void) { return 1; }
+extern "C" const char* moe_last_error(void) { return g_err; }
+
+namespace {
+
+__global__ void dense_offsets_kernel(int32_t* off, int M) {
+  if (threadIdx.x == 0) {
+    off[0] = 0;
+    off[1] = M;
+  }
+}
+
+struct Carver {
+  char* base;
+  size_t used;
+  void* take(size_t bytes) {
+    void* p = base ? base + used : nullptr;
+    used += (bytes + 255) & ~(size_t)255;
+    return p;
+  }
+};
+
+struct ForwardBuffers {
+  int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
+  float *w, *sx, *sh, *shs;
+  uint8_t *xq, *hq, *hsq;
+  void *y, *ys, *permute_ws, *gemm_ws;
+  size_t permute_ws_bytes, gemm_ws_bytes, total;
+};
+
+ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
+  ForwardBuffers b;
+  Carver c{(char*)ws, 0};
+  const size_t R = (size_t)M * k;
+  b.idx = (int32_t*)c.take(R * 4);
+  b.w = (float*)c.take(R * 4);
+  b.group_sizes = (int32_t*)c.take((size_t)E * 4);
+  b.group_offsets = (int32_t*)c.take((size_t)(E + 1) * 4);
+  b.sorted_token_ids = (int32_t*)c.take(R * 4);
+  b.inv_perm = (int32_t*)c.take(R * 4);
+  b.dense_off = (int32_t*)c.take(8);
+  b.permute_ws_bytes = moe_permute_workspace_bytes(M, k, E);
+  b.permute_ws = c.take(b.permute_ws_bytes);
+  size_t g1 = moe_gemm_workspace_bytes((int)R, E, I > D ? I : D);
+  size_t g2 = SI ? moe_gemm_workspace_bytes(M, 1, SI > D ? SI : D) : 0;
+  b.gemm_ws_bytes = g1 > g2 ? g1 : g2;
+  b.gemm_ws = c.take(b.gemm_ws_bytes);
+  b.xq = (uint8_t*)c.take((size_t)M * D);
+  b.sx = (float*)c.take((size_t)M * (D / 128) * 4);
+  b.hq = (uint8_t*)c.take(R * I);
+  b.sh = (float*)c.take(R * (I / 128) * 4);
+  b.y = c.take(R * D * 2);
+  b.hsq = SI ? (uint8_t*)c.take((size_t)M * SI) : nullptr;
+  b.shs = SI ? (float*)c.take((size_t)M * (SI / 128) * 4) : nullptr;
+  b.ys = SI ? c.take((size_t)M * D * 2) : nullptr;
+  b.total = c.used;
+  return b;
+}
+
+}  // namespace
+
+extern "C" size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI) {
+  if (M < 0 || D <= 0 || E <= 0 || k <= 0 || I <= 0 || SI < 0) return 0;
+  return carve(nullptr, M, D, E, k, I, SI).total;
+}
+
+extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, moe_stream_t stream) {
+  MOE_REQUIRE(a && ws, MOE_ERR_NULL, "forward: null args or workspace");
+  MOE_REQUIRE(a->M >= 0 && a->D > 0 && a->E >= 1 && a->k >= 1 && a->I > 0 && a->SI >= 0, MOE_ERR_BAD_SHAPE,
+              "forward: bad dims M=%d D=%d E=%d k=%d I=%d SI=%d", a->M, a->D, a->E, a->k, a->I, a->SI);
+  MOE_REQUIRE(a->D % 128 == 0 && a->I % 128 == 0 && a->SI % 128 == 0, MOE_ERR_BAD_SHAPE,
+              "forward: D=%d, I=%d and SI=%d must be multiples of 128", a->D, a->I, a->SI);
+  MOE_REQUIRE(a->x && a->logits && a->out && a->w_gate && a->w_up && a->w_down && a->sw_gate && a->sw_up && a->sw_down,
+              MOE_ERR_NULL, "forward: null tensor pointer");
+  if (a->SI)
+    MOE_REQUIRE(a->ws_gate && a->ws_up && a->ws_down && a->sws_gate && a->sws_up && a->sws_down, MOE_ERR_NULL,
+                "forward: SI > 0 but a shared-expert pointer is null");
+  MOE_REQUIRE(MOE_ALIGNED16(ws), MOE_ERR_BAD_ALIGN, "forward: workspace must be 16-byte aligned");
+  const size_t need = moe_forward_workspace_bytes(a->M, a->D, a->E, a->k, a->I, a->SI);
+  MOE_REQUIRE(ws_bytes >= need, MOE_ERR_WORKSPACE_TOO_SMALL, "forward: workspace %zu < %zu", ws_bytes, need);
+  if (a->M == 0) return MOE_OK;
+
+  ForwardBuffers b = carve(ws, a->M, a->D, a->E, a->k, a->I, a->SI);
+  int32_t* idx = a->out_idx ? a->out_idx : b.idx;
+  float* w = a->out_w ? a->out_w : b.w;
+  int32_t* gsz = a->out_group_sizes ? a->out_group_sizes : b.group_sizes;
+  int32_t* stid = a->out_sorted_token_ids ? a->out_sorted_token_ids : b.sorted_token_ids;
+  int32_t* inv = a->out_inv_perm ? a->out_inv_perm : b.inv_perm;
+  const int R = a->M * a->k;
+  int rc;
+  if (a->routing == MOE_ROUTING_SOFTMAX)
+    rc = moe_route_softmax_topk(a->logits, a->M, a->E, a->k, a->renorm, idx, w, stream);
+  else if (a->routing == MOE_ROUTING_SIGMOID_GROUPED)
+    rc = moe_route_sigmoid_grouped(a->logits, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
+                                   a->routed_scale, idx, w, stream);
+  else
+    return moe_set_error(MOE_ERR_BAD_SHAPE, "forward: unknown routing %d", a->routing);
+  if (rc) return rc;
+  if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
+                        b.permute_ws_bytes, stream)))
+    return rc;
+  if ((rc = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream))) return rc;
+  if ((rc = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets,
+                                       a->E, R, a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, stream)))
+    return rc;
+  if ((rc = moe_gemm_down_fp8(b.hq, b.sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
+                              b.gemm_ws, b.gemm_ws_bytes, stream)))
+    return rc;
+  if (a->SI) {
+    hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, b.dense_off, a->M);
+    if ((rc = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up,
+                                         b.dense_off, 1, a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws, b.gemm_ws_bytes,
+                                         stream)))
+      return rc;
+    if ((rc = moe_gemm_down_fp8(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
+                                b.gemm_ws, b.gemm_ws_bytes, stream)))
+      return rc;
+  }
+  return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, a->M, a->k, a->D, a->out, stream);
+}

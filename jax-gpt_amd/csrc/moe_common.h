@@ -1,0 +1,53 @@
+// Shared device/host helpers for the gfx950 MoE kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "moe_hip.h"
+
+#define MOE_WAVE 64
+#define MOE_QBLOCK 128  // scale granularity along K (and N for weights)
+#define MOE_FP8_MAX 448.0f
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef unsigned short bf16_t;  // raw bf16 bits
+
+// host side: record an error message for moe_last_error() and return the code
+int moe_set_error(int code, const char* fmt, ...);
+int moe_check_hip(hipError_t e, const char* what);
+
+#define MOE_REQUIRE(cond, code, ...) \
+  do {                               \
+    if (!(cond)) return moe_set_error(code, __VA_ARGS__); \
+  } while (0)
+#define MOE_ALIGNED16(p) ((((uintptr_t)(p)) & 15u) == 0)
+
+// ---- device helpers -------------------------------------------------------
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t b) { return __uint_as_float(((unsigned)b) << 16); }
+
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {  // round-to-nearest-even
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+// scale = 448/amax (1 when the group is all zero); both quotients are IEEE-rounded
+__device__ __forceinline__ void fp8_scales(float amax, float& scale, float& scale_inv) {
+  scale = amax > 0.f ? __fdiv_rn(MOE_FP8_MAX, amax) : 1.0f;
+  scale_inv = __fdiv_rn(1.0f, scale);
+}
+
+// four f32 -> four e4m3fn codes (RNE), clamped to +-448 first
+__device__ __forceinline__ unsigned pack4_e4m3(float a, float b, float c, float d) {
+  a = fminf(fmaxf(a, -MOE_FP8_MAX), MOE_FP8_MAX);
+  b = fminf(fmaxf(b, -MOE_FP8_MAX), MOE_FP8_MAX);
+  c = fminf(fmaxf(c, -MOE_FP8_MAX), MOE_FP8_MAX);
+  d = fminf(fmaxf(d, -MOE_FP8_MAX), MOE_FP8_MAX);
+  int v = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  v = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, v, true);
+  return (unsigned)v;
+}

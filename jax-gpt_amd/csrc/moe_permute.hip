@@ -1,0 +1,162 @@
+// Stable counting sort of the flat (token, slot) list by expert id.
+//
+// Replaces jax_gpt/models/qwen35/moe.py:58-80 (_sort_and_group: argsort of the
+// flat expert ids, the scatter-add histogram, and the gathers of token ids).
+// Three launches, all integer work:
+//   1. per-chunk histograms: each wavefront counts its 64 entries with ballot
+//      match masks and adds them to an LDS histogram of the chunk;
+//   2. one workgroup turns the (chunks x E) counts into group sizes, group
+//      offsets and, per chunk, the first output position of every expert;
+//   3. each chunk recomputes its entries' rank (earlier entries of the same
+//      expert: earlier waves via an LDS prefix, same wave via popcount of the
+//      match mask below the lane) and scatters.
+#include "moe_common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / MOE_WAVE;
+constexpr int kChunk = 2048;  // flat entries per workgroup
+constexpr int kRounds = kChunk / kThreads;
+constexpr int kMaxE = 1024;
+
+// lanes of this wave whose expert id equals mine (ids < 2^bits); inactive lanes pass id = -1
+__device__ __forceinline__ unsigned long long match_any(int id, int bits) {
+  unsigned long long m = __ballot(id >= 0);
+  for (int b = 0; b < bits; ++b) {
+    unsigned long long set = __ballot((id >> b) & 1);
+    m &= ((id >> b) & 1) ? set : ~set;
+  }
+  return id >= 0 ? m : 0ull;
+}
+
+__device__ __forceinline__ int ilog2_ceil(int n) {
+  int b = 0;
+  while ((1 << b) < n) ++b;
+  return b;
+}
+
+__global__ __launch_bounds__(kThreads) void hist_kernel(const int32_t* __restrict__ ids, int R, int E,
+                                                       int32_t* __restrict__ chunk_hist) {
+  extern __shared__ int hist[];  // E
+  for (int e = threadIdx.x; e < E; e += kThreads) hist[e] = 0;
+  __syncthreads();
+  const int bits = ilog2_ceil(E);
+  const int lane = threadIdx.x & 63;
+  const int base = blockIdx.x * kChunk;
+  for (int r = 0; r < kRounds; ++r) {
+    int f = base + r * kThreads + threadIdx.x;
+    int id = f < R ? ids[f] : -1;
+    if (id >= E) id = -1;  // out-of-range ids are dropped rather than corrupting LDS
+    unsigned long long m = match_any(id, bits);
+    // the lowest lane of each match class adds the class size
+    if (id >= 0 && (m & ((1ull << lane) - 1ull)) == 0ull) atomicAdd(&hist[id], __popcll(m));
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kThreads) chunk_hist[(size_t)blockIdx.x * E + e] = hist[e];
+}
+
+// one workgroup: thread e owns expert e (loop if E > blockDim)
+__global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk_hist, int n_chunks, int E,
+                                                    int32_t* __restrict__ group_sizes,
+                                                    int32_t* __restrict__ group_offsets) {
+  __shared__ int tot[kMaxE];
+  __shared__ int wave_tot[kMaxE / MOE_WAVE];
+  const int e = threadIdx.x;
+  int total = 0;
+  if (e < E) {
+    for (int c = 0; c < n_chunks; ++c) {  // exclusive scan down the chunks, in place
+      int v = chunk_hist[(size_t)c * E + e];
+      chunk_hist[(size_t)c * E + e] = total;
+      total += v;
+    }
+    group_sizes[e] = total;
+  }
+  // exclusive scan of totals over experts: wave scan + scan of wave totals
+  const int lane = e & 63, wv = e >> 6;
+  int incl = e < E ? total : 0;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    int o = __shfl_up(incl, off, MOE_WAVE);
+    if (lane >= off) incl += o;
+  }
+  if (lane == 63) wave_tot[wv] = incl;
+  __syncthreads();
+  int wbase = 0;
+  for (int i = 0; i < wv; ++i) wbase += wave_tot[i];
+  const int excl = wbase + incl - (e < E ? total : 0);
+  tot[e] = excl;
+  if (e < E) {
+    group_offsets[e] = excl;
+    if (e == E - 1) group_offsets[E] = excl + total;
+    for (int c = 0; c < n_chunks; ++c) chunk_hist[(size_t)c * E + e] += excl;  // absolute first position
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void scatter_kernel(const int32_t* __restrict__ ids, int R, int E, int k,
+                                                          const int32_t* __restrict__ chunk_base,
+                                                          int32_t* __restrict__ sorted_token_ids,
+                                                          int32_t* __restrict__ sort_order,
+                                                          int32_t* __restrict__ inv_perm) {
+  extern __shared__ int smem[];  // next[E]: next free output position per expert within this chunk
+  int* next = smem;
+  for (int e = threadIdx.x; e < E; e += kThreads) next[e] = chunk_base[(size_t)blockIdx.x * E + e];
+  __syncthreads();
+  const int bits = ilog2_ceil(E);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int base = blockIdx.x * kChunk;
+  for (int r = 0; r < kRounds; ++r) {
+    int f = base + r * kThreads + threadIdx.x;
+    int id = f < R ? ids[f] : -1;
+    if (id >= E) id = -1;  // out-of-range ids are dropped rather than corrupting LDS
+    unsigned long long m = match_any(id, bits);
+    int rank = __popcll(m & ((1ull << lane) - 1ull));
+    int cnt = __popcll(m);
+    // waves take their turn in flat-index order so ranks stay stable
+    int pos = 0;
+    for (int turn = 0; turn < kWaves; ++turn) {
+      if (wv == turn && id >= 0) {
+        pos = next[id] + rank;  // every lane of a class reads before its leader bumps the counter
+      }
+      __syncthreads();
+      if (wv == turn && id >= 0 && rank == 0) next[id] += cnt;
+      __syncthreads();
+    }
+    if (id >= 0) {
+      if (sort_order) sort_order[pos] = f;
+      if (sorted_token_ids) sorted_token_ids[pos] = f / k;
+      if (inv_perm) inv_perm[f] = pos;
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" size_t moe_permute_workspace_bytes(int M, int k, int E) {
+  long long R = (long long)M * k;
+  long long chunks = (R + kChunk - 1) / kChunk;
+  if (chunks < 1) chunks = 1;
+  return (size_t)(chunks * E * sizeof(int32_t) + 256);
+}
+
+extern "C" int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* group_sizes,
+                           int32_t* group_offsets, int32_t* sorted_token_ids, int32_t* sort_order,
+                           int32_t* inv_perm, void* ws, size_t ws_bytes, moe_stream_t stream) {
+  MOE_REQUIRE(idx && group_sizes && group_offsets && ws, MOE_ERR_NULL, "permute: null pointer");
+  MOE_REQUIRE(M >= 0 && k >= 1 && E >= 1 && E <= kMaxE, MOE_ERR_BAD_SHAPE,
+              "permute: need k >= 1 and 1 <= E <= %d, got M=%d k=%d E=%d", kMaxE, M, k, E);
+  MOE_REQUIRE((long long)M * k < (1ll << 31), MOE_ERR_BAD_SHAPE, "permute: M*k overflows int32");
+  MOE_REQUIRE(ws_bytes >= moe_permute_workspace_bytes(M, k, E), MOE_ERR_WORKSPACE_TOO_SMALL,
+              "permute: workspace %zu < %zu", ws_bytes, moe_permute_workspace_bytes(M, k, E));
+  hipStream_t s = (hipStream_t)stream;
+  const int R = M * k;
+  int n_chunks = (R + kChunk - 1) / kChunk;
+  if (n_chunks < 1) n_chunks = 1;
+  int32_t* chunk_hist = (int32_t*)ws;
+  hipLaunchKernelGGL(hist_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, chunk_hist);
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kMaxE), 0, s, chunk_hist, n_chunks, E, group_sizes, group_offsets);
+  if (R > 0 && (sorted_token_ids || sort_order || inv_perm))
+    hipLaunchKernelGGL(scatter_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, k,
+                       chunk_hist, sorted_token_ids, sort_order, inv_perm);
+  return moe_check_hip(hipGetLastError(), "permute launch");
+}

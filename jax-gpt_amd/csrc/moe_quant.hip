@@ -1,0 +1,98 @@
+// Block-scaled e4m3fn quantisers (HBM-bound, 16-byte accesses).
+//
+// scale = 448/amax, q = e4m3(clamp(x*scale, +-448)), stored scale = 1/scale.
+// Activations: 1x128 groups (replaces the per-row quantiser of
+// jax_gpt/models/qwen35/fp8.py:30-45).  Weights: 128x128 blocks in the
+// (E, out, in) layout of quantize.py:31-42.
+#include "moe_common.h"
+
+namespace {
+
+struct alignas(16) bf16x8 { bf16_t v[8]; };
+
+// 16 lanes per 128-wide group, 8 bf16 (16 B) per lane
+__global__ __launch_bounds__(256) void quant_act_kernel(const bf16x8* __restrict__ x, long long n_pieces,
+                                                       int groups_per_row, uint2* __restrict__ xq,
+                                                       float* __restrict__ sx) {
+  long long p = (long long)blockIdx.x * 256 + threadIdx.x;
+  bool ok = p < n_pieces;
+  bf16x8 in = {};
+  if (ok) in = x[p];
+  float f[8], amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    f[i] = bf16_to_f32(in.v[i]);
+    amax = fmaxf(amax, fabsf(f[i]));
+  }
+#pragma unroll
+  for (int off = 1; off < 16; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, MOE_WAVE));
+  float scale, scale_inv;
+  fp8_scales(amax, scale, scale_inv);
+  if (ok) {
+    uint2 out;
+    out.x = pack4_e4m3(f[0] * scale, f[1] * scale, f[2] * scale, f[3] * scale);
+    out.y = pack4_e4m3(f[4] * scale, f[5] * scale, f[6] * scale, f[7] * scale);
+    xq[p] = out;
+    if ((threadIdx.x & 15) == 0) sx[p >> 4] = scale_inv;
+  }
+}
+
+// one workgroup per 128x128 block; thread t reads row t/2, columns (t%2)*64 .. +64
+template <typename T>
+__global__ __launch_bounds__(256) void quant_weight_kernel(const T* __restrict__ w, int N, int K,
+                                                          uint8_t* __restrict__ wq, float* __restrict__ sw) {
+  __shared__ float red[4];
+  const int kb = blockIdx.x, nb = blockIdx.y, e = blockIdx.z;
+  const int row = nb * 128 + (threadIdx.x >> 1);
+  const int col = kb * 128 + (threadIdx.x & 1) * 64;
+  const size_t off = ((size_t)e * N + row) * K + col;
+  float f[64];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 64; ++i) {
+    if constexpr (sizeof(T) == 2) f[i] = bf16_to_f32(((const bf16_t*)w)[off + i]);
+    else f[i] = ((const float*)w)[off + i];
+    amax = fmaxf(amax, fabsf(f[i]));
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, MOE_WAVE));
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = amax;
+  __syncthreads();
+  amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float scale, scale_inv;
+  fp8_scales(amax, scale, scale_inv);
+  unsigned* out = (unsigned*)(wq + off);
+#pragma unroll
+  for (int i = 0; i < 16; ++i)
+    out[i] = pack4_e4m3(f[4 * i] * scale, f[4 * i + 1] * scale, f[4 * i + 2] * scale, f[4 * i + 3] * scale);
+  if (threadIdx.x == 0) sw[((size_t)e * (N / 128) + nb) * (K / 128) + kb] = scale_inv;
+}
+
+}  // namespace
+
+extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream) {
+  MOE_REQUIRE(x_bf16 && xq && sx, MOE_ERR_NULL, "quant_act: null pointer");
+  MOE_REQUIRE(R >= 0 && K > 0 && K % MOE_QBLOCK == 0, MOE_ERR_BAD_SHAPE, "quant_act: K=%d must be a positive multiple of 128 (R=%d)", K, R);
+  MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(xq), MOE_ERR_BAD_ALIGN, "quant_act: pointers must be 16-byte aligned");
+  if (R == 0) return MOE_OK;
+  long long pieces = (long long)R * K / 8;
+  long long blocks = (pieces + 255) / 256;
+  MOE_REQUIRE(blocks < (1ll << 31), MOE_ERR_BAD_SHAPE, "quant_act: too many elements");
+  hipLaunchKernelGGL(quant_act_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const bf16x8*)x_bf16, pieces, K / 128, (uint2*)xq, sx);
+  return moe_check_hip(hipGetLastError(), "quant_act launch");
+}
+
+extern "C" int moe_quant_weight_block(const void* w, int src_is_f32, int E, int N, int K, uint8_t* wq,
+                                      float* sw, moe_stream_t stream) {
+  MOE_REQUIRE(w && wq && sw, MOE_ERR_NULL, "quant_weight_block: null pointer");
+  MOE_REQUIRE(E >= 1 && N > 0 && K > 0 && N % 128 == 0 && K % 128 == 0 && E < 65536 && N / 128 < 65536,
+              MOE_ERR_BAD_SHAPE, "quant_weight_block: N=%d and K=%d must be multiples of 128 (E=%d)", N, K, E);
+  MOE_REQUIRE(MOE_ALIGNED16(w) && MOE_ALIGNED16(wq), MOE_ERR_BAD_ALIGN, "quant_weight_block: pointers must be 16-byte aligned");
+  dim3 grid(K / 128, N / 128, E);
+  if (src_is_f32)
+    hipLaunchKernelGGL(quant_weight_kernel<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float*)w, N, K, wq, sw);
+  else
+    hipLaunchKernelGGL(quant_weight_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)w, N, K, wq, sw);
+  return moe_check_hip(hipGetLastError(), "quant_weight_block launch");
+}

@@ -1,0 +1,338 @@
+"""Host side of the MoE expert forward: the reference's call surface over the C ABI.
+
+Mirrors jax_gpt/models/qwen35/moe.py -- `moe_routing` (:37), `_sort_and_group`
+(:58, here `permute`), `expert_forward_single` (:97), `shared_expert_forward`
+(:225) and `moe_layer` (:235) -- with torch CUDA tensors as the device buffers
+and the current torch stream as the HIP stream.  All arithmetic happens in
+libmoe_hip.so; torch only allocates.
+
+Expert weights are block-scaled fp8 dicts ``{'w': (E, out, in) float8_e4m3fn,
+'scale_inv': (E, out/128, in/128) float32}`` -- the reference's fp8 layout
+(quantize.py:31-42, model.py:89-97) with 128x128 scale blocks instead of
+per-row scales; real value = w * scale_inv (moe.py:29).  Plain (E, in, out)
+arrays, the reference's unquantised layout, are quantised on the GPU on first
+use.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import weakref
+
+import torch
+
+from ._lib import MoeForwardArgs, check, lib
+
+ROUTING = {"softmax": 0, "sigmoid_grouped": 1}
+
+
+# ----------------------------------------------------------------------------
+# plumbing
+# ----------------------------------------------------------------------------
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(0) if t is None else C.c_void_p(t.data_ptr())
+
+
+def _dev(t, dtype=None, name="tensor"):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch.Tensor, got {type(t).__name__}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name}: must live on the GPU (this path has no CPU fallback)")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    return t.contiguous()
+
+
+def _codes(t, name):
+    """fp8 weights/activations travel as bytes; accept float8_e4m3fn or uint8."""
+    if t.dtype == torch.float8_e4m3fn:
+        t = t.view(torch.uint8)
+    return _dev(t, torch.uint8, name)
+
+
+def _empty(shape, dtype, like):
+    return torch.empty(shape, dtype=dtype, device=like.device)
+
+
+# ----------------------------------------------------------------------------
+# routing (moe.py:37-55) and the DeepSeek-V3 group-limited router
+# ----------------------------------------------------------------------------
+
+def route_softmax_topk(logits, k, renorm=True):
+    logits = _dev(logits, torch.float32, "logits")
+    M, E = logits.shape
+    idx = _empty((M, k), torch.int32, logits)
+    w = _empty((M, k), torch.float32, logits)
+    check(lib().moe_route_softmax_topk(_ptr(logits), M, E, k, int(renorm), _ptr(idx), _ptr(w), _stream()))
+    return idx, w
+
+
+def route_sigmoid_grouped(logits, bias, n_group, topk_group, k, renorm=True, routed_scale=1.0):
+    logits = _dev(logits, torch.float32, "logits")
+    bias = None if bias is None else _dev(bias, torch.float32, "bias")
+    M, E = logits.shape
+    if bias is not None and tuple(bias.shape) != (E,):
+        raise ValueError(f"bias: expected shape ({E},), got {tuple(bias.shape)}")
+    idx = _empty((M, k), torch.int32, logits)
+    w = _empty((M, k), torch.float32, logits)
+    check(lib().moe_route_sigmoid_grouped(_ptr(logits), _ptr(bias), M, E, n_group, topk_group, k, int(renorm),
+                                          float(routed_scale), _ptr(idx), _ptr(w), _stream()))
+    return idx, w
+
+
+# ----------------------------------------------------------------------------
+# sort / group (moe.py:58-80)
+# ----------------------------------------------------------------------------
+
+def permute(expert_indices, n_experts):
+    """Stable sort of the flat (token, slot) list by expert.  Returns a dict with
+    group_sizes (E,), group_offsets (E+1,), sorted_token_ids, sort_order, inv_perm (R,)."""
+    idx = _dev(expert_indices, torch.int32, "expert_indices")
+    M, k = idx.shape
+    R = M * k
+    out = dict(group_sizes=_empty((n_experts,), torch.int32, idx),
+               group_offsets=_empty((n_experts + 1,), torch.int32, idx),
+               sorted_token_ids=_empty((R,), torch.int32, idx),
+               sort_order=_empty((R,), torch.int32, idx),
+               inv_perm=_empty((R,), torch.int32, idx))
+    nbytes = lib().moe_permute_workspace_bytes(M, k, n_experts)
+    ws = _empty((nbytes,), torch.uint8, idx)
+    check(lib().moe_permute(_ptr(idx), M, k, n_experts, _ptr(out["group_sizes"]), _ptr(out["group_offsets"]),
+                            _ptr(out["sorted_token_ids"]), _ptr(out["sort_order"]), _ptr(out["inv_perm"]),
+                            _ptr(ws), nbytes, _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------
+# quantisers
+# ----------------------------------------------------------------------------
+
+def quant_act(x):
+    """(R, K) bf16 -> (codes (R, K) float8_e4m3fn, scale_inv (R, K/128) f32)."""
+    x = _dev(x, torch.bfloat16, "x")
+    R, K = x.shape
+    xq = _empty((R, K), torch.uint8, x)
+    sx = _empty((R, K // 128), torch.float32, x)
+    check(lib().moe_quant_act(_ptr(x), R, K, _ptr(xq), _ptr(sx), _stream()))
+    return xq.view(torch.float8_e4m3fn), sx
+
+
+def quantize_weight_block(w):
+    """(E, out, in) or (out, in) bf16/f32 -> {'w': float8_e4m3fn, 'scale_inv': f32 (.., out/128, in/128)}.
+
+    The block-scaled counterpart of the reference's `_quantize_weight`
+    (quantize.py:18-42); the input is already in (out, in) order."""
+    if w.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"weights must be bf16 or f32, got {w.dtype}")
+    w = _dev(w, None, "w")
+    squeeze = w.dim() == 2
+    w3 = w.unsqueeze(0) if squeeze else w
+    E, N, K = w3.shape
+    wq = _empty((E, N, K), torch.uint8, w)
+    sw = _empty((E, N // 128, K // 128), torch.float32, w)
+    check(lib().moe_quant_weight_block(_ptr(w3), int(w.dtype == torch.float32), E, N, K, _ptr(wq), _ptr(sw),
+                                       _stream()))
+    if squeeze:
+        wq, sw = wq[0], sw[0]
+    return {"w": wq.view(torch.float8_e4m3fn), "scale_inv": sw}
+
+
+_plain_cache = {}
+
+
+def _expert_weight(w, name):
+    """Accept a block-fp8 dict, or a plain (E, in, out) array as the reference stores
+    unquantised experts (model.py:98-101), which is transposed and quantised once."""
+    if isinstance(w, dict) and "w" in w:
+        q, s = w["w"], w["scale_inv"]
+        if q.dim() == 2:
+            q, s = q.unsqueeze(0), s.unsqueeze(0)
+        E, N, K = q.shape
+        if tuple(s.shape) != (E, N // 128, K // 128):
+            raise ValueError(
+                f"{name}: scale_inv has shape {tuple(s.shape)}; this path needs 128x128 block scales "
+                f"{(E, N // 128, K // 128)} (per-row scales of the reference's quantize.py must be re-quantised "
+                "with quantize_weight_block)")
+        return _codes(q, name + "['w']"), _dev(s, torch.float32, name + "['scale_inv']")
+    if not isinstance(w, torch.Tensor):
+        raise TypeError(f"{name}: expected a tensor or an fp8 dict")
+    key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
+    hit = _plain_cache.get(key)
+    if hit is not None and hit[0]() is w:
+        return hit[1], hit[2]
+    w3 = w.unsqueeze(0) if w.dim() == 2 else w
+    if w3.dtype not in (torch.bfloat16, torch.float32):
+        w3 = w3.to(torch.float32)
+    d = quantize_weight_block(w3.transpose(-1, -2).contiguous())      # (E, in, out) -> (E, out, in)
+    q, s = d["w"].view(torch.uint8), d["scale_inv"]
+    _plain_cache[key] = (weakref.ref(w), q, s)
+    return q, s
+
+
+# ----------------------------------------------------------------------------
+# grouped GEMMs (moe.py:83-87) and combine (moe.py:90-94)
+# ----------------------------------------------------------------------------
+
+def _gemm_ws(R, E, n_out, like):
+    nbytes = lib().moe_gemm_workspace_bytes(R, E, n_out)
+    return _empty((nbytes,), torch.uint8, like), nbytes
+
+
+def gemm_gateup_swiglu(xq, sx, gate, up, group_offsets, row_ids=None, n_rows=None):
+    """h = silu(x.Wg^T) * (x.Wu^T) per expert row range, quantised 1x128 -> (hq, sh).
+    row_ids maps sorted position -> row of xq (None: rows are already in expert order)."""
+    xq = _codes(xq, "xq")
+    sx = _dev(sx, torch.float32, "sx")
+    wg, sg = _expert_weight(gate, "gate_proj")
+    wu, su = _expert_weight(up, "up_proj")
+    E, I, D = wg.shape
+    if wu.shape != wg.shape or xq.shape[1] != D:
+        raise ValueError(f"shape mismatch: x {tuple(xq.shape)}, gate {tuple(wg.shape)}, up {tuple(wu.shape)}")
+    go = _dev(group_offsets, torch.int32, "group_offsets")
+    if go.numel() != E + 1:
+        raise ValueError(f"group_offsets needs {E + 1} entries, got {go.numel()}")
+    if row_ids is not None:
+        row_ids = _dev(row_ids, torch.int32, "row_ids")
+        R = row_ids.numel() if n_rows is None else n_rows
+    else:
+        R = xq.shape[0] if n_rows is None else n_rows
+    hq = _empty((R, I), torch.uint8, xq)
+    sh = _empty((R, I // 128), torch.float32, xq)
+    ws, nbytes = _gemm_ws(R, E, I, xq)
+    check(lib().moe_gemm_gateup_swiglu_fp8(_ptr(xq), _ptr(sx), _ptr(row_ids), _ptr(wg), _ptr(sg), _ptr(wu), _ptr(su),
+                                           _ptr(go), E, R, D, I, _ptr(hq), _ptr(sh), _ptr(ws), nbytes, _stream()))
+    return hq.view(torch.float8_e4m3fn), sh
+
+
+def gemm_down(hq, sh, down, group_offsets):
+    """y = h . Wdown[e]^T per expert row range, bf16 (R, D)."""
+    hq = _codes(hq, "hq")
+    sh = _dev(sh, torch.float32, "sh")
+    wd, sd = _expert_weight(down, "down_proj")
+    E, D, I = wd.shape
+    R = hq.shape[0]
+    if hq.shape[1] != I:
+        raise ValueError(f"shape mismatch: h {tuple(hq.shape)}, down {tuple(wd.shape)}")
+    go = _dev(group_offsets, torch.int32, "group_offsets")
+    y = _empty((R, D), torch.bfloat16, hq)
+    ws, nbytes = _gemm_ws(R, E, D, hq)
+    check(lib().moe_gemm_down_fp8(_ptr(hq), _ptr(sh), _ptr(wd), _ptr(sd), _ptr(go), E, R, I, D, _ptr(y), _ptr(ws),
+                                  nbytes, _stream()))
+    return y
+
+
+def combine(y, weights, inv_perm, shared=None):
+    y = _dev(y, torch.bfloat16, "y")
+    weights = _dev(weights, torch.float32, "weights")
+    inv_perm = _dev(inv_perm, torch.int32, "inv_perm")
+    shared = None if shared is None else _dev(shared, torch.bfloat16, "shared")
+    M, k = weights.shape
+    D = y.shape[1]
+    out = _empty((M, D), torch.bfloat16, y)
+    check(lib().moe_combine(_ptr(y), _ptr(weights), _ptr(inv_perm), _ptr(shared), M, k, D, _ptr(out), _stream()))
+    return out
+
+
+# ----------------------------------------------------------------------------
+# the reference's functions
+# ----------------------------------------------------------------------------
+
+def expert_forward_single(x, expert_indices, expert_weights, gate_proj, up_proj, down_proj):
+    """moe.py:97-114: sort/group, grouped SwiGLU, weighted scatter back.  x (M, D) bf16."""
+    x = _dev(x, torch.bfloat16, "x")
+    wg, _ = _expert_weight(gate_proj, "gate_proj")
+    E = wg.shape[0]
+    sg = permute(expert_indices, E)
+    xq, sx = quant_act(x)
+    hq, sh = gemm_gateup_swiglu(xq, sx, gate_proj, up_proj, sg["group_offsets"], row_ids=sg["sorted_token_ids"])
+    y = gemm_down(hq, sh, down_proj, sg["group_offsets"])
+    return combine(y, expert_weights, sg["inv_perm"])
+
+
+def shared_expert_forward(x, gate_proj, up_proj, down_proj):
+    """moe.py:225-232: dense SwiGLU MLP on every token (one group holding all rows)."""
+    x = _dev(x, torch.bfloat16, "x")
+    M = x.shape[0]
+    off = torch.tensor([0, M], dtype=torch.int32, device=x.device)
+    xq, sx = quant_act(x)
+    hq, sh = gemm_gateup_swiglu(xq, sx, gate_proj, up_proj, off)
+    return gemm_down(hq, sh, down_proj, off)
+
+
+def moe_routing(x, gate_weight, n_experts_per_token):
+    """moe.py:37-55.  The router matmul is not part of this path yet: pass router
+    logits to `moe_experts`, or logits computed by the caller."""
+    raise NotImplementedError(
+        "moe_routing(x, gate_weight, k) needs the router matmul, which this build does not provide yet; "
+        "call route_softmax_topk(router_logits, k) or moe_experts(x, router_logits, ...)")
+
+
+def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=None, n_group=1, topk_group=1,
+                renorm=True, routed_scale=1.0, shared=None, return_debug=False):
+    """Router logits in, combined hidden states out (one C-ABI call, `moe_forward`).
+
+    x (M, D) bf16; router_logits (M, E) f32; experts / shared: dicts with keys
+    'gate_proj', 'up_proj', 'down_proj' holding block-fp8 dicts (or plain arrays).
+    Returns (M, D) bf16, plus a dict of the integer intermediates if return_debug."""
+    x = _dev(x, torch.bfloat16, "x")
+    logits = _dev(router_logits, torch.float32, "router_logits")
+    if routing not in ROUTING:
+        raise ValueError(f"routing must be one of {sorted(ROUTING)}, got {routing!r}")
+    M, D = x.shape
+    wg, sg = _expert_weight(experts["gate_proj"], "gate_proj")
+    wu, su = _expert_weight(experts["up_proj"], "up_proj")
+    wd, sd = _expert_weight(experts["down_proj"], "down_proj")
+    E, I, _ = wg.shape
+    if tuple(logits.shape) != (M, E):
+        raise ValueError(f"router_logits: expected {(M, E)}, got {tuple(logits.shape)}")
+    if wg.shape != (E, I, D) or wu.shape != (E, I, D) or wd.shape != (E, D, I):
+        raise ValueError(f"expert weight shapes {tuple(wg.shape)} {tuple(wu.shape)} {tuple(wd.shape)} do not fit D={D}")
+    a = MoeForwardArgs()
+    a.M, a.D, a.E, a.k, a.I = M, D, E, top_k, I
+    a.routing, a.n_group, a.topk_group, a.renorm, a.routed_scale = ROUTING[routing], n_group, topk_group, int(renorm), routed_scale
+    keep = [x, logits, wg, sg, wu, su, wd, sd]
+    a.x, a.logits = x.data_ptr(), logits.data_ptr()
+    if bias is not None:
+        bias = _dev(bias, torch.float32, "bias")
+        keep.append(bias)
+        a.bias = bias.data_ptr()
+    a.w_gate, a.w_up, a.w_down = wg.data_ptr(), wu.data_ptr(), wd.data_ptr()
+    a.sw_gate, a.sw_up, a.sw_down = sg.data_ptr(), su.data_ptr(), sd.data_ptr()
+    SI = 0
+    if shared is not None:
+        swg, ssg = _expert_weight(shared["gate_proj"], "shared gate_proj")
+        swu, ssu = _expert_weight(shared["up_proj"], "shared up_proj")
+        swd, ssd = _expert_weight(shared["down_proj"], "shared down_proj")
+        SI = swg.shape[1]
+        if swg.shape != (1, SI, D) or swu.shape != (1, SI, D) or swd.shape != (1, D, SI):
+            raise ValueError("shared expert weight shapes do not fit")
+        keep += [swg, ssg, swu, ssu, swd, ssd]
+        a.ws_gate, a.ws_up, a.ws_down = swg.data_ptr(), swu.data_ptr(), swd.data_ptr()
+        a.sws_gate, a.sws_up, a.sws_down = ssg.data_ptr(), ssu.data_ptr(), ssd.data_ptr()
+    a.SI = SI
+    out = _empty((M, D), torch.bfloat16, x)
+    a.out = out.data_ptr()
+    dbg = None
+    if return_debug:
+        R = M * top_k
+        dbg = dict(indices=_empty((M, top_k), torch.int32, x), weights=_empty((M, top_k), torch.float32, x),
+                   group_sizes=_empty((E,), torch.int32, x), sorted_token_ids=_empty((R,), torch.int32, x),
+                   inv_perm=_empty((R,), torch.int32, x))
+        a.out_idx, a.out_w = dbg["indices"].data_ptr(), dbg["weights"].data_ptr()
+        a.out_group_sizes = dbg["group_sizes"].data_ptr()
+        a.out_sorted_token_ids, a.out_inv_perm = dbg["sorted_token_ids"].data_ptr(), dbg["inv_perm"].data_ptr()
+    nbytes = lib().moe_forward_workspace_bytes(M, D, E, top_k, I, SI)
+    ws = _empty((max(nbytes, 16),), torch.uint8, x)
+    check(lib().moe_forward(C.byref(a), _ptr(ws), nbytes, _stream()))
+    del keep
+    return (out, dbg) if return_debug else out
+
+
+def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=None):
+    """moe.py:235-282.  Needs the router matmul (see moe_routing)."""
+    raise NotImplementedError("moe_layer needs the router matmul, which this build does not provide yet; "
+                              "use moe_experts(x, router_logits, ...)")
