@@ -1,0 +1,230 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE expert forward path on one MI355X.
+
+A step is one pass of the whole path (router logits in, combined hidden states
+out: routing, permute, activation quantisation, both grouped fp8 GEMMs, shared
+expert, combine) over one batch of synthetic input that is already resident in
+HBM.  The headline workload is the DeepSeek-V3-style prefill layer; the same
+run also measures the decode shape (HBM-bound) and reports it under "decode".
+
+Prints ONE JSON line.  FLOPs counted: 6*R*D*I (routed) + 6*M*D*SI (shared); the
+router matmul and tile padding are not counted.  Decode bytes counted: fp8
+weights (and their scales) of the experts actually touched plus the shared
+expert; activations are not counted.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0     # MI355X dense fp8 MFMA (published)
+PEAK_HBM_GBS = 8000.0        # MI355X HBM3E (published)
+
+WORKLOADS = {
+    # BASELINE config 3 / 4: DeepSeek-V3-style layer
+    "deepseek_v3_prefill": dict(M=8192, D=7168, E=256, k=8, I=2048, SI=2048, routing="sigmoid_grouped",
+                                n_group=8, topk_group=4),
+    "deepseek_v3_decode": dict(M=64, D=7168, E=256, k=8, I=2048, SI=2048, routing="sigmoid_grouped",
+                               n_group=8, topk_group=4),
+    # BASELINE config 2: Qwen3-MoE-style layer
+    "qwen3_moe_prefill": dict(M=4096, D=2048, E=128, k=8, I=768, SI=0, routing="softmax", n_group=1, topk_group=1),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_weights(jg, torch, E, N, K, gen, std=0.02, chunk=16):
+    """(E, N, K) N(0, std) weights, block-quantised on the GPU chunk by chunk (never on the host)."""
+    wq = torch.empty((E, N, K), dtype=torch.float8_e4m3fn, device="cuda")
+    sw = torch.empty((E, N // 128, K // 128), dtype=torch.float32, device="cuda")
+    for e0 in range(0, E, chunk):
+        n = min(chunk, E - e0)
+        w = (torch.randn((n, N, K), dtype=torch.float32, device="cuda", generator=gen) * std).to(torch.bfloat16)
+        d = jg.quantize_weight_block(w)
+        wq[e0:e0 + n] = d["w"]
+        sw[e0:e0 + n] = d["scale_inv"]
+        del w, d
+    return {"w": wq, "scale_inv": sw}
+
+
+def make_layer(jg, torch, cfg, seed=0):
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    D, E, I, SI = cfg["D"], cfg["E"], cfg["I"], cfg["SI"]
+    experts = dict(gate_proj=make_weights(jg, torch, E, I, D, gen), up_proj=make_weights(jg, torch, E, I, D, gen),
+                   down_proj=make_weights(jg, torch, E, D, I, gen))
+    shared = None
+    if SI:
+        shared = dict(gate_proj=make_weights(jg, torch, 1, SI, D, gen), up_proj=make_weights(jg, torch, 1, SI, D, gen),
+                      down_proj=make_weights(jg, torch, 1, D, SI, gen))
+    bias = None
+    if cfg["routing"] == "sigmoid_grouped":
+        bias = torch.randn((E,), dtype=torch.float32, device="cuda", generator=gen) * 0.1
+    return experts, shared, bias, gen
+
+
+def make_inputs(torch, cfg, gen):
+    x = torch.randn((cfg["M"], cfg["D"]), dtype=torch.float32, device="cuda", generator=gen).to(torch.bfloat16)
+    logits = torch.randn((cfg["M"], cfg["E"]), dtype=torch.float32, device="cuda", generator=gen)
+    return x, logits
+
+
+def timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return start.elapsed_time(stop) / steps, wall
+
+
+def run_workload(jg, torch, name, cfg, layer, steps, warmup):
+    experts, shared, bias, gen = layer
+    x, logits = make_inputs(torch, cfg, gen)
+    kw = dict(top_k=cfg["k"], experts=experts, shared=shared, routing=cfg["routing"], bias=bias,
+              n_group=cfg["n_group"], topk_group=cfg["topk_group"])
+    out, dbg = jg.moe_experts(x, logits, return_debug=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all(), "non-finite output"
+    gs = dbg["group_sizes"].cpu()
+    touched = int((gs > 0).sum())
+    assert int(gs.sum()) == cfg["M"] * cfg["k"]
+    ev_ms, wall_ms = timed(torch, lambda: jg.moe_experts(x, logits, **kw), steps, warmup)
+    M, D, E, k, I, SI = (cfg[n] for n in ("M", "D", "E", "k", "I", "SI"))
+    R = M * k
+    flops = 6.0 * R * D * I + 6.0 * M * D * SI
+    per_expert_bytes = 3 * D * I + 3 * (D // 128) * (I // 128) * 4
+    shared_bytes = (3 * D * SI + 3 * (D // 128) * (SI // 128) * 4) if SI else 0
+    weight_bytes = touched * per_expert_bytes + shared_bytes
+    res = dict(workload=name, ms_per_step=ev_ms, wall_ms_per_step=wall_ms, flops=flops, tflops=flops / ev_ms / 1e9,
+               touched_experts=touched, weight_bytes=weight_bytes, gbs=weight_bytes / ev_ms / 1e6)
+
+    # the dominant kernel alone: the gate/up grouped GEMM (routed launch + shared launch), HIP events on the
+    # stream it is launched on (torch's current stream is the stream handed to the C ABI)
+    sg = jg.permute(dbg["indices"], E)
+    xq, sx = jg.quant_act(x)
+    dense_off = torch.tensor([0, M], dtype=torch.int32, device="cuda")
+
+    def gateup():
+        jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], sg["group_offsets"],
+                              row_ids=sg["sorted_token_ids"])
+        if shared:
+            jg.gemm_gateup_swiglu(xq, sx, shared["gate_proj"], shared["up_proj"], dense_off)
+
+    n_launch = 2 if shared else 1
+    k_ms, _ = timed(torch, gateup, steps, max(2, warmup // 2))
+    k_flops = 4.0 * R * D * I + 4.0 * M * D * SI
+    res["gateup_kernel"] = dict(avg_launch_ms=k_ms / n_launch, flops_per_launch=k_flops / n_launch,
+                                tflops=k_flops / k_ms / 1e9, launches_per_step=n_launch)
+    k_bytes = touched * per_expert_bytes * 2 / 3 + (shared_bytes * 2 / 3)
+    res["gateup_kernel"]["gbs"] = k_bytes / k_ms / 1e6
+    res["gateup_kernel"]["bytes_per_launch"] = k_bytes / n_launch
+    return res
+
+
+def cpu_baseline(cfg, seconds_budget=25.0):
+    """The reference's dataflow (oracle/reference_dataflow.py, a port) on the host cores, on a bounded
+    sample of the prefill workload: a few experts at their mean row count."""
+    import torch
+    from oracle import reference_dataflow as RD
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)                  # a one-GPU box gives this job 16 cores' worth
+    rows = max(cfg["M"] * cfg["k"] // cfg["E"], 1)
+    n_exp = 4
+    t0 = time.perf_counter()
+    r = RD.time_expert_sample(cfg["D"], cfg["I"], n_exp, rows, top_k=cfg["k"], reps=3, threads=threads)
+    log(f"cpu baseline: {r['sample']}: {r['seconds']:.2f} s/pass, total {time.perf_counter() - t0:.1f} s")
+    return {"value": r["flops"] / r["seconds"] / 1e12, "unit": "TFLOP/s", "cores": r["cores"], "kind": "port",
+            "sample": r["sample"]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="deepseek_v3_prefill", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (expert parallelism is shown as one "
+              "GPU's shard); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import jax_gpt_amd as jg
+    from jax_gpt_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    jg.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+
+    cfg = WORKLOADS[args.workload]
+    t0 = time.perf_counter()
+    layer = make_layer(jg, torch, cfg)
+    torch.cuda.synchronize()
+    log(f"weights for {args.workload} generated in {time.perf_counter() - t0:.1f} s")
+    main_res = run_workload(jg, torch, args.workload, cfg, layer, args.steps, args.warmup)
+    log(json.dumps(main_res))
+    is_decode = args.workload.endswith("decode")
+
+    decode = None
+    if not is_decode and not args.no_decode and args.workload == "deepseek_v3_prefill":
+        dcfg = WORKLOADS["deepseek_v3_decode"]
+        decode = run_workload(jg, torch, "deepseek_v3_decode", dcfg, layer, max(args.steps, 20), args.warmup)
+        log(json.dumps(decode))
+
+    gk = main_res["gateup_kernel"]
+    if is_decode:
+        metric, value, unit = "MoE layer HBM GB/s over touched fp8 expert weights (decode)", main_res["gbs"], "GB/s"
+        roof = {"bound": "hbm", "achieved": gk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": gk["gbs"] / PEAK_HBM_GBS, "traffic": None, "kernel": "gate/up grouped GEMM",
+                "avg_launch_ms": gk["avg_launch_ms"]}
+    else:
+        metric, value, unit = "MoE layer fp8 TFLOP/s (prefill)", main_res["tflops"], "TFLOP/s"
+        roof = {"bound": "mfma", "achieved": gk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": None, "kernel": "grouped_gemm_kernel<0> (gate/up + SwiGLU)",
+                "avg_launch_ms": gk["avg_launch_ms"], "flops_per_launch": gk["flops_per_launch"]}
+    line = {
+        "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3", "data": "synthetic",
+        "config": {"workload": args.workload, **{k: cfg[k] for k in ("M", "D", "E", "k", "I", "SI", "routing")},
+                   "touched_experts": main_res["touched_experts"]},
+        "frac_of_peak": (value / PEAK_HBM_GBS) if is_decode else (value / PEAK_FP8_TFLOPS),
+        "roofline": roof,
+    }
+    if decode:
+        dk = decode["gateup_kernel"]
+        line["decode"] = {"metric": "HBM GB/s over touched fp8 expert weights", "value": decode["gbs"], "unit": "GB/s",
+                          "ms_per_step": decode["ms_per_step"], "touched_experts": decode["touched_experts"],
+                          "weight_bytes": decode["weight_bytes"], "frac_of_peak": decode["gbs"] / PEAK_HBM_GBS,
+                          "roofline": {"bound": "hbm", "achieved": dk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                       "frac": dk["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                                       "avg_launch_ms": dk["avg_launch_ms"]}}
+    if not args.no_cpu:
+        pcfg = cfg if not is_decode else WORKLOADS["deepseek_v3_prefill"]
+        line["cpu_baseline"] = cpu_baseline(pcfg)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
