@@ -6,42 +6,48 @@
 //   MODE_DOWN:   y = h . Wdown[e]^T, bf16
 // for the rows [group_offsets[e], group_offsets[e+1]) of every expert e.
 //
-// Shape of the computation.  Both operands are K-contiguous e4m3 with one f32
-// scale per 128 K-elements (activations: per row; weights: per 128 rows), so
-// one v_mfma_f32_16x16x128_f8f6f4 consumes exactly one scale block: its 16x16
-// f32 result is a partial sum that is multiplied by sx[row,kb]*sw[nblk,kb] and
-// added to the f32 accumulator on the vector ALU.  The weight fragment is the
-// MFMA's row operand and the activation fragment its column operand, so a lane
-// holds four weight rows of ONE activation row: one activation scale per lane
-// per fragment instead of four.
+// Arithmetic.  Both operands are K-contiguous e4m3 with one f32 scale per 128
+// K-elements (activations: per row; weights: per 128 rows), so one
+// v_mfma_f32_16x16x128_f8f6f4 consumes exactly one scale block: its 16x16 f32
+// result is a partial sum that is multiplied by sx[row,kb]*sw[nblk,kb] and
+// added to the f32 accumulator on the vector ALU (the matrix unit has no f32
+// scale input).  The weight fragment is the MFMA's row operand and the
+// activation fragment its column operand, so a lane holds four weight rows of
+// ONE activation row: one activation scale per lane per fragment, not four.
 //
-// Tiling.  A workgroup (4 waves) owns a work item = (expert, <=128 activation
-// rows, 256 weight rows) and walks K in steps of 128 with two LDS buffers.
-// In MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of
-// the same output columns, so silu(g)*u and the 1x128 amax stay inside the
-// workgroup.  Wave w owns weight rows {32w..32w+31} of each half (GATEUP) or
-// {64w..64w+63} (DOWN) against all 128 activation rows: 4x8 MFMA tiles.
-// LDS rows are 128 B; 16-byte chunks are XOR-swizzled with (row & 7) so that
-// both the cooperative tile stores and the per-lane fragment reads are
-// conflict-free.  Work items are listed on the device by build_items_kernel
-// (no host read-back of group sizes) in [expert][column block][row tile] order
-// and dealt to the 8 XCDs in contiguous ranges, so the row tiles that share a
-// weight slab run together under one L2.
+// Data movement.  A workgroup (8 waves, two per SIMD) owns a work item =
+// (expert, <= 128 activation rows, 256 weight rows) and walks K in steps of 128
+// through a ring of three LDS stages.  Tiles are copied global -> LDS by
+// global_load_lds (no registers in between), two steps ahead of the MFMAs.
+// In MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of the
+// same output columns, so silu(g)*u is lane-local and the 1x128 amax stays
+// inside the workgroup.  Waves form a 4 x 2 grid: wave (wi, xj) owns weight rows
+// {32wi..32wi+31} of each half (GATEUP) or {64wi..64wi+63} (DOWN) against
+// activation rows [64 xj, 64 xj + 64): 4x4 MFMA tiles, 64 accumulator registers.
+//
+// Work items are listed on the device by build_items_kernel (no host read-back
+// of group sizes) in [expert][column block][row tile] order and dealt to the 8
+// XCDs in contiguous ranges, so the row tiles and column blocks that share a
+// weight slab or an activation tile run together under one L2.
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "moe_common.h"
 
 namespace {
 
-constexpr int BM = 128;       // activation rows per work item
 constexpr int BW = 256;       // weight rows per work item
+constexpr int BM = 128;       // activation rows per work item
 constexpr int BK = 128;       // K step = scale block
-constexpr int NT = 256;       // threads
+constexpr int NWAVES = 8;
+constexpr int NT = 64 * NWAVES;
 constexpr int MODE_GATEUP = 0;
 constexpr int MODE_DOWN = 1;
 
-constexpr int W_TILE_BYTES = BW * BK;   // 32 KB
-constexpr int X_TILE_BYTES = BM * BK;   // 16 KB
-constexpr int BUF_BYTES = W_TILE_BYTES + X_TILE_BYTES + BM * 4;  // + activation scales
-constexpr int LDS_BYTES = 2 * BUF_BYTES;
+#ifndef MOE_VAR
+#define MOE_VAR 0   // development switch: bit 0 = no scale FMA, bit 1 = no copies in the loop
+#endif
 
 struct WorkHeader {
   int n_items;
@@ -53,9 +59,9 @@ struct WorkItem {
 
 // ---- work list -----------------------------------------------------------
 
-// One workgroup.  tiles[e] = ceil(rows_e / BM); item order [expert][col_block][row tile].
+// One workgroup.  tiles[e] = ceil(rows_e / bm); item order [expert][col_block][row tile].
 __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __restrict__ group_offsets, int E,
-                                                          int n_col_blocks, int max_items,
+                                                          int n_col_blocks, int bm, int max_items,
                                                           WorkHeader* __restrict__ hdr, WorkItem* __restrict__ items) {
   __shared__ int tile_prefix[1025];
   __shared__ int wave_tot[16];
@@ -63,7 +69,7 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
   const int lane = e & 63, wv = e >> 6;
   int rows = 0;
   if (e < E) rows = group_offsets[e + 1] - group_offsets[e];
-  int tiles = rows > 0 ? (rows + BM - 1) / BM : 0;
+  int tiles = rows > 0 ? (rows + bm - 1) / bm : 0;
   int incl = tiles;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -81,14 +87,12 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
   if (total > max_items) total = max_items;  // cannot happen for consistent offsets; keeps writes in bounds
   if (e == 0) hdr->n_items = total;
   for (int it = threadIdx.x; it < total; it += blockDim.x) {
-    const int tile_major = it / n_col_blocks;  // which expert: search on tile_prefix * n_col_blocks
     // find expert x with tile_prefix[x]*ncb <= it < tile_prefix[x+1]*ncb
-    int lo = 0, hi = E;  // invariant: tile_prefix[lo]*ncb <= it < tile_prefix[hi]*ncb
+    int lo = 0, hi = E;
     while (hi - lo > 1) {
       int mid = (lo + hi) >> 1;
       if (tile_prefix[mid] * n_col_blocks <= it) lo = mid; else hi = mid;
     }
-    (void)tile_major;
     const int x = lo;
     const int tiles_x = tile_prefix[x + 1] - tile_prefix[x];
     const int local = it - tile_prefix[x] * n_col_blocks;
@@ -96,19 +100,56 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
     const int start = group_offsets[x], rows_x = group_offsets[x + 1] - start;
     WorkItem w;
     w.expert = x;
-    w.row_start = start + rt * BM;
-    w.row_count = min(BM, rows_x - rt * BM);
+    w.row_start = start + rt * bm;
+    w.row_count = min(bm, rows_x - rt * bm);
     w.col_block = cb;
     items[it] = w;
   }
 }
 
 // ---- main kernel ---------------------------------------------------------
+//
+// LDS stage = [weight tile 256 x 128 B][activation tile 128 x 128 B][128 activation scales].
+// Tiles are row-major with 128-byte rows; the 16-byte chunk c of row r sits at chunk position
+// c ^ ((r >> 1) & 7).  A fragment lane (row fr = lane % 16, quarter fq = lane / 16) feeds the
+// MFMA with K bytes [16 fq, +16) and [64 + 16 fq, +16) of its row -- the same choice for both
+// operands, so the contraction is unchanged -- which makes every ds_read_b128 of a fragment
+// conflict-free (measured ~240 B/clk/CU against ~125 B/clk for 32 contiguous bytes per lane).
+// global_load_lds_dwordx4 writes LDS base + lane * 16, i.e. one wave instruction fills 8
+// consecutive tile rows; the swizzle is applied by choosing which 16-byte piece of the row
+// each lane fetches.  No asynchronous load ever targets a register.
 
+constexpr int NSTAGE = 3;
+constexpr int W_TILE_BYTES = BW * BK;              // 32 KB
+constexpr int X_TILE_BYTES = BM * BK;              // 16 KB
+constexpr int STAGE_X_OFF = W_TILE_BYTES;
+constexpr int STAGE_S_OFF = W_TILE_BYTES + X_TILE_BYTES;
+constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4;  // 49664
+constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;    // 148992
+constexpr int VM_PER_STEP = 7;                     // per wave per K step: 4 weight + 2 activation + 1 scale copy
+
+// epilogue staging tile: 128-byte rows, chunk c of row r at position c ^ (r & 7)
 __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 4); }
 
+// The copies are inline assembly on purpose: when the compiler knows that an instruction writes LDS from
+// memory it makes every later LDS read wait for ALL outstanding memory operations, which would empty the
+// prefetch queue at every K step.  Completion is tracked by hand instead (wait_vm + barrier); these are the
+// only vector-memory operations inside the K loop.  The LDS destination of lane l is m0 + l * size.
+__device__ __forceinline__ void dma16(const uint8_t* g, uint8_t* l) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(const float* g, uint8_t* l) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void wait_vm() {
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));   // vmcnt = N, other counters untouched
+}
+
 template <int MODE>
-__global__ __launch_bounds__(NT) void grouped_gemm_kernel(
+__global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0,   // gate (GATEUP) or down (DOWN)
     const uint8_t* __restrict__ w1, const float* __restrict__ sw1,   // up (GATEUP only)
@@ -125,139 +166,159 @@ __global__ __launch_bounds__(NT) void grouped_gemm_kernel(
   if (slot >= per_xcd || item_id >= n_items) return;
   const WorkItem item = items[item_id];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wi = wave & 3, xj = wave >> 2;
+  const int fr = lane & 15, fq = lane >> 4;
   const int KB = K / BK;
-  const int nkb_scale = KB;  // scale columns per weight row block
   const int e = item.expert;
-
-  // weight rows of this item: GATEUP -> rows [cb*128, +128) of gate and of up; DOWN -> rows [cb*256, +256) of down
   const int wrow0 = MODE == MODE_GATEUP ? item.col_block * 128 : item.col_block * 256;
-  const uint8_t* wbase0 = w0 + ((size_t)e * N) * K;
-  const uint8_t* wbase1 = MODE == MODE_GATEUP ? w1 + ((size_t)e * N) * K : nullptr;
 
-  // ---- per-thread global sources for the cooperative tile loads (16 B each)
-  const int ld_chunk = tid & 7, ld_row = tid >> 3;  // rows ld_row + 32*i
-  const uint8_t* wsrc[8];
+  // ---- copy sources.  Wave w fills 1 KB row groups [4w, 4w+4) of the weight tile, [2w, 2w+2) of the
+  // activation tile and scale slots [16w, 16w+16).
+  const int drow = lane >> 3, dchunk = lane & 7;
+  const uint8_t* wsrc[4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    int r = ld_row + 32 * i;  // 0..255 within the weight tile
+  for (int i = 0; i < 4; ++i) {
+    const int r = (wave * 4 + i) * 8 + drow;                   // row within the 256-row weight tile
+    const int piece = dchunk ^ ((r >> 1) & 7);
     const uint8_t* base;
     int grow;
     if (MODE == MODE_GATEUP) {
-      base = r < 128 ? wbase0 : wbase1;
+      base = r < 128 ? w0 : w1;
       grow = wrow0 + (r & 127);
     } else {
-      base = wbase0;
+      base = w0;
       grow = min(wrow0 + r, N - 1);
     }
-    wsrc[i] = base + (size_t)grow * K + ld_chunk * 16;
+    wsrc[i] = base + ((size_t)e * N + grow) * K + piece * 16;
   }
-  const uint8_t* xsrc[4];
+  const uint8_t* xsrc[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int r = min(ld_row + 32 * i, item.row_count - 1);
-    int g = item.row_start + r;
+  for (int i = 0; i < 2; ++i) {
+    const int r = (wave * 2 + i) * 8 + drow;                   // row within the activation tile
+    const int piece = dchunk ^ ((r >> 1) & 7);
+    int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
-    xsrc[i] = xq + (size_t)g * K + ld_chunk * 16;
+    xsrc[i] = xq + (size_t)g * K + piece * 16;
   }
-  const float* sxsrc = nullptr;
-  if (tid < BM) {
-    int g = item.row_start + min(tid, item.row_count - 1);
+  // scale slot 64 h + fr * 4 + j holds the scale of tile row 64 h + 16 j + fr: a lane reads its 4 scales as 16 bytes
+  const float* ssrc;
+  {
+    const int p = wave * 16 + (lane & 15);
+    const int q = p & 63;
+    const int r = (p & 64) + 16 * (q & 3) + (q >> 2);
+    int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
-    sxsrc = sx + (size_t)g * KB;
+    ssrc = sx + (size_t)g * KB;
   }
-  // weight scale rows for this wave
+  auto issue = [&](int kb) {   // VM_PER_STEP operations
+    uint8_t* st = lds + (kb % NSTAGE) * STAGE_BYTES;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(wsrc[i] + (size_t)kb * BK, st + (wave * 4 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) dma16(xsrc[i] + (size_t)kb * BK, st + STAGE_X_OFF + (wave * 2 + i) * 1024);
+    if (lane < 16) dma4(ssrc + kb, st + STAGE_S_OFF + wave * 64);
+  };
+
+  // weight scales of this wave's rows
   const float* swp0;
   const float* swp1 = nullptr;
   if (MODE == MODE_GATEUP) {
-    swp0 = sw0 + ((size_t)e * (N / 128) + item.col_block) * nkb_scale;
-    swp1 = sw1 + ((size_t)e * (N / 128) + item.col_block) * nkb_scale;
+    swp0 = sw0 + ((size_t)e * (N / 128) + item.col_block) * KB;
+    swp1 = sw1 + ((size_t)e * (N / 128) + item.col_block) * KB;
   } else {
-    int nb = min(item.col_block * 2 + (wave >> 1), N / 128 - 1);
-    swp0 = sw0 + ((size_t)e * (N / 128) + nb) * nkb_scale;
+    const int nb = min(item.col_block * 2 + (wi >> 1), N / 128 - 1);
+    swp0 = sw0 + ((size_t)e * (N / 128) + nb) * KB;
   }
 
-  v4i wreg[8], xreg[4];
-  float sxreg = 0.f;
-  auto load_tile = [&](int kb) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) wreg[i] = *(const v4i*)(wsrc[i] + (size_t)kb * BK);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) xreg[i] = *(const v4i*)(xsrc[i] + (size_t)kb * BK);
-    if (tid < BM) sxreg = sxsrc[kb];
-  };
-  auto store_tile = [&](int buf) {
-    uint8_t* wl = lds + buf * BUF_BYTES;
-    uint8_t* xl = wl + W_TILE_BYTES;
-    float* sl = (float*)(xl + X_TILE_BYTES);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *(v4i*)(wl + swz(ld_row + 32 * i, ld_chunk)) = wreg[i];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(v4i*)(xl + swz(ld_row + 32 * i, ld_chunk)) = xreg[i];
-    if (tid < BM) sl[tid] = sxreg;
-  };
-
-  // ---- fragment geometry
-  const int fr = lane & 15;        // row of the fragment this lane feeds
-  const int fq = lane >> 4;        // K quarter (32 B) this lane feeds
-  int wfrag_row[4];
+  const int lane_off0 = fr * BK + ((fq ^ (fr >> 1)) << 4);         // K bytes [16 fq, +16)
+  const int lane_off1 = fr * BK + (((fq + 4) ^ (fr >> 1)) << 4);   // K bytes [64 + 16 fq, +16)
+  int wfrag_off[4];                                                // byte offset of each weight fragment in the stage
 #pragma unroll
   for (int f = 0; f < 4; ++f)
-    wfrag_row[f] = MODE == MODE_GATEUP ? ((f >> 1) * 128 + wave * 32 + (f & 1) * 16 + fr) : (wave * 64 + f * 16 + fr);
+    wfrag_off[f] = (MODE == MODE_GATEUP ? ((f >> 1) * 128 + wi * 32 + (f & 1) * 16) : (wi * 64 + f * 16)) * BK;
+  // activation fragments past the item's last row are never multiplied (uniform per wave)
+  const int jmax = min(4, max(0, (item.row_count - xj * 64 + 15) >> 4));
 
-  v4f acc[4][8];
+  v4f acc[4][4];
 #pragma unroll
   for (int f = 0; f < 4; ++f)
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[f][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j) acc[f][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
+  issue(0);
+  if (KB > 1) issue(1);
+  float s0n = swp0[0], s1n = MODE == MODE_GATEUP ? swp1[0] : 0.f;
 
   for (int kb = 0; kb < KB; ++kb) {
-    const int buf = kb & 1;
-    if (kb + 1 < KB) load_tile(kb + 1);
-
-    const uint8_t* wl = lds + buf * BUF_BYTES;
-    const uint8_t* xl = wl + W_TILE_BYTES;
-    const float* sl = (const float*)(xl + X_TILE_BYTES);
-    const float s0 = swp0[kb];
-    const float s1 = MODE == MODE_GATEUP ? swp1[kb] : s0;
-
-    v8i wf[4];
-#pragma unroll
-    for (int f = 0; f < 4; ++f) {
-      v4i lo = *(const v4i*)(wl + swz(wfrag_row[f], 2 * fq));
-      v4i hi = *(const v4i*)(wl + swz(wfrag_row[f], 2 * fq + 1));
-      wf[f] = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    // stage kb has landed once only the next step's copies are still outstanding
+    if (MOE_VAR & 2) {
+    } else if (kb + 1 < KB) {
+      wait_vm<VM_PER_STEP>();
+    } else {
+      wait_vm<0>();
     }
+    __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; stage (kb-1) % NSTAGE is free again
+    if (!(MOE_VAR & 2) && kb + 2 < KB) issue(kb + 2);
+
+    const uint8_t* st = lds + (kb % NSTAGE) * STAGE_BYTES;
+    const float s0 = s0n, s1 = MODE == MODE_GATEUP ? s1n : s0n;
+    if (kb + 1 < KB) {   // next step's weight scales, one step early
+      s0n = swp0[kb + 1];
+      if (MODE == MODE_GATEUP) s1n = swp1[kb + 1];
+    }
+    auto read_frag = [&](const uint8_t* base) {
+      const v4i lo = *(const v4i*)(base + lane_off0);
+      const v4i hi = *(const v4i*)(base + lane_off1);
+      return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    };
+    const uint8_t* xt = st + STAGE_X_OFF + xj * 64 * BK;
+    v8i wf[4], xf[4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int xr = j * 16 + fr;
-      v4i lo = *(const v4i*)(xl + swz(xr, 2 * fq));
-      v4i hi = *(const v4i*)(xl + swz(xr, 2 * fq + 1));
-      v8i xf = (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-      const float sxv = sl[xr];
-      const float sc0 = sxv * s0, sc1 = sxv * s1;
+    for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
 #pragma unroll
-      for (int f = 0; f < 4; ++f) {
-        v4f p = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-        const float sc = (MODE == MODE_GATEUP && f >= 2) ? sc1 : sc0;
-        acc[f][j] += p * sc;
+    for (int j = 0; j < 4; ++j) xf[j] = read_frag(xt + j * 16 * BK);
+    float sc0[4], sc1[4];
+    {
+      const v4f a = *(const v4f*)(st + STAGE_S_OFF + xj * 256 + fr * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        sc0[j] = a[j] * s0;
+        sc1[j] = a[j] * s1;
       }
     }
-    if (kb + 1 < KB) store_tile(buf ^ 1);
-    __syncthreads();
-  }
-
-  // ---- epilogue.  Lane holds, for fragment (f, j): activation row j*16+fr, weight rows (fragment base)+4*fq+{0..3}.
-  if (MODE == MODE_GATEUP) {
-    float* amax_s = (float*)lds;                       // [4 waves][128 rows]
-    uint8_t* tile = lds + 4 * BM * sizeof(float);      // [128 rows][128 B], swizzled
-    float amax[8];
+    // one uniform branch per K step: the common full tile runs a branch-free schedule
+    auto mma = [&](auto full) {
+      constexpr bool FULL = decltype(full)::value;
+      v4f p[2][4];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j <= 4; ++j) {
+        if (j < 4 && (FULL || j < jmax)) {
+#pragma unroll
+          for (int f = 0; f < 4; ++f)
+            if (MOE_VAR & 1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf[j], acc[f][j], 0, 0, 0, 0, 0, 0);
+            else p[j & 1][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf[j], (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+        }
+        if (!(MOE_VAR & 1) && j > 0 && (FULL || j - 1 < jmax)) {
+          const int jj = j - 1;
+#pragma unroll
+          for (int f = 0; f < 4; ++f)
+            acc[f][jj] += p[jj & 1][f] * ((MODE == MODE_GATEUP && f >= 2) ? sc1[jj] : sc0[jj]);
+        }
+      }
+    };
+    if (jmax == 4) mma(std::true_type{});
+    else mma(std::false_type{});
+  }
+  __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
+
+  // ---- epilogue.  Lane holds, for fragment (f, j): tile row xj*64 + j*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
+  if (MODE == MODE_GATEUP) {
+    float* amax_s = (float*)lds;                       // [4 weight-wave groups][128 rows]
+    uint8_t* tile = lds + 4 * BM * sizeof(float);      // [128 rows][128 B], swizzled
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
       float m = 0.f;
 #pragma unroll
       for (int f = 0; f < 2; ++f)
@@ -270,31 +331,31 @@ __global__ __launch_bounds__(NT) void grouped_gemm_kernel(
         }
       m = fmaxf(m, __shfl_xor(m, 16, MOE_WAVE));
       m = fmaxf(m, __shfl_xor(m, 32, MOE_WAVE));
-      amax[j] = m;
-      if (fq == 0) amax_s[wave * BM + j * 16 + fr] = m;
+      if (fq == 0) amax_s[wi * BM + xj * 64 + j * 16 + fr] = m;
     }
     __syncthreads();
     const int I = N;
     uint8_t* hq = (uint8_t*)out;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int xr = j * 16 + fr;
+    for (int j = 0; j < 4; ++j) {
+      const int xr = xj * 64 + j * 16 + fr;
       float m = fmaxf(fmaxf(amax_s[xr], amax_s[BM + xr]), fmaxf(amax_s[2 * BM + xr], amax_s[3 * BM + xr]));
       float scale, scale_inv;
       fp8_scales(m, scale, scale_inv);
 #pragma unroll
       for (int f = 0; f < 2; ++f) {
         unsigned q = pack4_e4m3(acc[f][j][0] * scale, acc[f][j][1] * scale, acc[f][j][2] * scale, acc[f][j][3] * scale);
-        const int col = wave * 32 + f * 16 + fq * 4;  // byte column within the 128-wide slab
+        const int col = wi * 32 + f * 16 + fq * 4;  // byte column within the 128-wide slab
         *(unsigned*)(tile + swz(xr, col >> 4) + (col & 15)) = q;
       }
-      if (wave == 0 && fq == 0 && xr < item.row_count)
+      if (wi == 0 && fq == 0 && xr < item.row_count)
         out_scale[(size_t)(item.row_start + xr) * (I / 128) + item.col_block] = scale_inv;
     }
     __syncthreads();
+    const int ld_chunk = tid & 7, ld_row = tid >> 3;   // 64 rows per pass
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = ld_row + 32 * i;
+    for (int i = 0; i < 2; ++i) {
+      const int r = ld_row + 64 * i;
       if (r < item.row_count) {
         v4i v = *(const v4i*)(tile + swz(r, ld_chunk));
         *(v4i*)(hq + (size_t)(item.row_start + r) * I + item.col_block * 128 + ld_chunk * 16) = v;
@@ -304,11 +365,11 @@ __global__ __launch_bounds__(NT) void grouped_gemm_kernel(
     // bf16 tile [128 rows][256 cols] = 512 B per row, 32 chunks of 16 B, swizzled with (row & 7)
     uint8_t* tile = lds;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int xr = j * 16 + fr;
+    for (int j = 0; j < 4; ++j) {
+      const int xr = xj * 64 + j * 16 + fr;
 #pragma unroll
       for (int f = 0; f < 4; ++f) {
-        const int col = wave * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
+        const int col = wi * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
         uint2 v;
         v.x = (unsigned)f32_to_bf16(acc[f][j][0]) | ((unsigned)f32_to_bf16(acc[f][j][1]) << 16);
         v.y = (unsigned)f32_to_bf16(acc[f][j][2]) | ((unsigned)f32_to_bf16(acc[f][j][3]) << 16);
@@ -318,11 +379,11 @@ __global__ __launch_bounds__(NT) void grouped_gemm_kernel(
     }
     __syncthreads();
     bf16_t* y = (bf16_t*)out;
-    const int c32 = tid & 31, r8 = tid >> 5;
+    const int c32 = tid & 31, r16 = tid >> 5;          // 16 rows per pass
     const int ncols = min(256, N - wrow0);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int r = r8 + 8 * i;
+    for (int i = 0; i < 8; ++i) {
+      const int r = r16 + 16 * i;
       if (r < item.row_count && c32 * 8 < ncols) {
         v4i v = *(const v4i*)(tile + r * 512 + ((c32 ^ (r & 7)) << 4));
         *(v4i*)(y + (size_t)(item.row_start + r) * N + wrow0 + c32 * 8) = v;
@@ -340,24 +401,24 @@ template <int MODE>
 int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
            const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
            void* out, float* out_scale, void* ws, size_t ws_bytes, hipStream_t s) {
-  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
   const size_t need = moe_gemm_workspace_bytes(R, E, N);
   MOE_REQUIRE(ws_bytes >= need, MOE_ERR_WORKSPACE_TOO_SMALL, "gemm: workspace %zu < %zu", ws_bytes, need);
   if (R == 0) return MOE_OK;
+  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
   const int max_items = max_items_for(R, E, ncb);
   WorkHeader* hdr = (WorkHeader*)ws;
   WorkItem* items = (WorkItem*)((char*)ws + sizeof(WorkHeader));
-  hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, ncb, max_items, hdr, items);
-  static bool attr_set[2] = {false, false};
-  if (!attr_set[MODE]) {
+  hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, ncb, BM, max_items, hdr, items);
+  static bool attr_set = false;
+  if (!attr_set) {
     hipError_t err = hipFuncSetAttribute((const void*)grouped_gemm_kernel<MODE>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (err != hipSuccess) return moe_check_hip(err, "gemm: raising the dynamic LDS limit");
-    attr_set[MODE] = true;
+    attr_set = true;
   }
   const int grid = ((max_items + 7) / 8) * 8;
-  hipLaunchKernelGGL(grouped_gemm_kernel<MODE>, dim3(grid), dim3(NT), LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1,
-                     sw1, hdr, items, K, N, out, out_scale);
+  hipLaunchKernelGGL(grouped_gemm_kernel<MODE>, dim3(grid), dim3(NT), LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1, sw1,
+                     hdr, items, K, N, out, out_scale);
   return moe_check_hip(hipGetLastError(), "gemm launch");
 }
 
