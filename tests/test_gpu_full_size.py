@@ -1,0 +1,177 @@
+"""Parity at the benchmark configurations' full sizes (BASELINE configs 2-5).
+
+The oracle cannot run these sizes in full, so each test checks
+  * every integer result (routing indices, group sizes, permutation) exactly against
+    the oracle, which is cheap at any size;
+  * the bf16 output on a sample of token rows against the oracle's per-row path
+    (weights of the sampled tokens' experts are copied back from the GPU);
+  * size-independent properties: a sub-batch gives bit-identical rows; every routed
+    row is written exactly once; empty experts are skipped.
+Weights are generated on the GPU (the DeepSeek-V3 shape is 11.3 GB of fp8) by the same
+quantiser whose bit-exactness the small tests pin."""
+import numpy as np
+import pytest
+
+from oracle import moe_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    import jax_gpt_amd as jg
+    import bench
+    jg.lib()
+    return jg, torch, bench
+
+
+def _fetch(experts):
+    """fetch(e) -> oracle-style dict for one expert, copied back from the GPU."""
+    import torch
+
+    def f(e):
+        out = {}
+        for name, key in (("gate", "gate_proj"), ("up", "up_proj"), ("down", "down_proj")):
+            q = experts[key]["w"][e].view(torch.uint8).cpu().numpy()
+            s = experts[key]["scale_inv"][e].cpu().numpy()
+            out[name] = (q, s)
+        return out
+    return f
+
+
+def _check_layer(jg, torch, cfg, layer, seed, n_sample):
+    experts, shared, bias, _ = layer
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    M, D, E, k, I = cfg["M"], cfg["D"], cfg["E"], cfg["k"], cfg["I"]
+    x = torch.randn((M, D), dtype=torch.float32, device="cuda", generator=gen).to(torch.bfloat16)
+    logits = torch.randn((M, E), dtype=torch.float32, device="cuda", generator=gen)
+    kw = dict(top_k=k, experts=experts, shared=shared, routing=cfg["routing"], bias=bias,
+              n_group=cfg["n_group"], topk_group=cfg["topk_group"])
+    out, dbg = jg.moe_experts(x, logits, return_debug=True, **kw)
+    torch.cuda.synchronize()
+
+    # integers: exact
+    lg = logits.cpu().numpy()
+    if cfg["routing"] == "softmax":
+        ridx, rw = O.route_softmax_topk(lg, k)
+    else:
+        ridx, rw = O.route_sigmoid_grouped(lg, None if bias is None else bias.cpu().numpy(), cfg["n_group"],
+                                           cfg["topk_group"], k)
+    assert np.array_equal(dbg["indices"].cpu().numpy(), ridx)
+    assert np.allclose(dbg["weights"].cpu().numpy(), rw, rtol=2e-6, atol=1e-9)
+    sg = O.sort_and_group(ridx, E)
+    assert np.array_equal(dbg["group_sizes"].cpu().numpy(), sg["group_sizes"])
+    assert np.array_equal(dbg["sorted_token_ids"].cpu().numpy(), sg["sorted_token_ids"])
+    assert np.array_equal(dbg["inv_perm"].cpu().numpy(), sg["inv_perm"])
+    assert int(sg["group_sizes"].sum()) == M * k
+    _say("   experts touched:", int((sg["group_sizes"] > 0).sum()), "largest group:", int(sg["group_sizes"].max()))
+
+    # sampled rows against the oracle
+    outn = H.bf16_to_np(out)
+    assert np.isfinite(outn).all()
+    rng = H.rng_for(seed)
+    tokens = sorted(set([0, M - 1] + list(rng.integers(0, M, n_sample - 2))))
+    xs = H.bf16_to_np(x[torch.tensor(tokens, device="cuda")])
+    xfull = np.zeros((max(tokens) + 1, D), np.float32)
+    xfull[tokens] = xs
+    sh = None
+    if shared is not None:
+        f = _fetch(shared)(0)
+        sh = {n: (q[None], s[None]) for n, (q, s) in f.items()}
+    want = O.moe_experts_rows(xfull, tokens, ridx, rw, _fetch(experts), shared=sh)
+    err = H.assert_close_out(outn[tokens], want, tol=1e-2, inner=I)
+    _say(f"   {len(tokens)} sampled rows: max-normalised error {err:.2e}")
+
+    # a sub-batch gives the same rows, bit for bit (a row's arithmetic does not depend on its tile)
+    nsub = min(M, 96)
+    part = jg.moe_experts(x[:nsub].contiguous(), logits[:nsub].contiguous(), **kw)
+    assert torch.equal(out[:nsub], part)
+    return out
+
+
+def test_config2_qwen3_moe_prefill(env):
+    jg, torch, bench = env
+    _say("config 2: Qwen3-MoE-style prefill")
+    cfg = bench.WORKLOADS["qwen3_moe_prefill"]
+    layer = bench.make_layer(jg, torch, cfg, seed=2)
+    _check_layer(jg, torch, cfg, layer, seed=20, n_sample=16)
+
+
+@pytest.fixture(scope="module")
+def dsv3_layer(env):
+    jg, torch, bench = env
+    return bench.make_layer(jg, torch, bench.WORKLOADS["deepseek_v3_prefill"], seed=3)
+
+
+def test_config3_deepseek_v3_prefill(env, dsv3_layer):
+    jg, torch, bench = env
+    _say("config 3: DeepSeek-V3-style prefill")
+    _check_layer(jg, torch, bench.WORKLOADS["deepseek_v3_prefill"], dsv3_layer, seed=30, n_sample=4)
+
+
+def test_config4_deepseek_v3_decode(env, dsv3_layer):
+    jg, torch, bench = env
+    _say("config 4: DeepSeek-V3-style decode")
+    _check_layer(jg, torch, bench.WORKLOADS["deepseek_v3_decode"], dsv3_layer, seed=40, n_sample=4)
+
+
+def test_config5_expert_parallel_shard_skewed(env):
+    """One GPU's expert-parallel shard: 32 local experts of the DeepSeek-V3 shape, 16384 pre-dispatched rows in
+    expert order with Zipf(1.2) group sizes (some experts empty), top-8 weights from Dirichlet(1), 2048 tokens."""
+    jg, torch, bench = env
+    _say("config 5: expert-parallel shard, skewed")
+    E, D, I, k, M = 32, 7168, 2048, 8, 2048
+    R = M * k
+    rng = H.rng_for(5)
+    p = 1.0 / np.arange(1, E + 1) ** 1.2
+    p[[5, 17, 30]] = 0.0                                       # forced empty experts
+    p /= p.sum()
+    rows_expert = np.sort(rng.choice(E, size=R, p=p))          # pre-dispatched: rows already in expert order
+    group_sizes = np.bincount(rows_expert, minlength=E).astype(np.int32)
+    assert (group_sizes == 0).sum() >= 3
+    off = np.concatenate([[0], np.cumsum(group_sizes)]).astype(np.int32)
+    weights = rng.dirichlet(np.ones(k), size=M).astype(np.float32)
+    inv_perm = rng.permutation(R).astype(np.int32)             # token slot (t, s) -> its row in the dispatched buffer
+
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    experts = dict(gate_proj=bench.make_weights(jg, torch, E, I, D, gen), up_proj=bench.make_weights(jg, torch, E, I, D, gen),
+                   down_proj=bench.make_weights(jg, torch, E, D, I, gen))
+    xs = torch.randn((R, D), dtype=torch.float32, device="cuda", generator=gen).to(torch.bfloat16)
+    xq, sx = jg.quant_act(xs)
+    d_off = H.to_cuda(off)
+    hq, sh = jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], d_off)
+    y = torch.full((R, D), float("nan"), dtype=torch.bfloat16, device="cuda")
+    y = jg.gemm_down(hq, sh, experts["down_proj"], d_off)
+    out = jg.combine(y, H.to_cuda(weights), H.to_cuda(inv_perm))
+    torch.cuda.synchronize()
+    yn = H.bf16_to_np(y)
+    assert np.isfinite(yn).all() and np.isfinite(H.bf16_to_np(out)).all()
+
+    # sampled dispatched rows (first/last row of the biggest and the smallest non-empty groups, and random ones)
+    fetch = _fetch(experts)
+    nz = np.nonzero(group_sizes)[0]
+    big, small = nz[np.argmax(group_sizes[nz])], nz[np.argmin(group_sizes[nz])]
+    rows = sorted(set([int(off[big]), int(off[big + 1] - 1), int(off[small]), int(off[small + 1] - 1)] + list(rng.integers(0, R, 4))))
+    xsn = H.bf16_to_np(xs[torch.tensor(rows, device="cuda")])
+    want = []
+    for i, r in enumerate(rows):
+        e = int(rows_expert[r])
+        ex = {n: (q[None], s[None]) for n, (q, s) in fetch(e).items()}
+        q1, s1 = O.quant_act_group(xsn[i:i + 1])
+        yy, _, _ = O.expert_swiglu(q1, s1, ex, np.array([0, 1], np.int32))
+        want.append(yy[0])
+    err = H.assert_close_out(yn[rows], np.stack(want), tol=1e-2, inner=I)
+    _say(f"   {len(rows)} sampled rows: max-normalised error {err:.2e}; group sizes min/max {group_sizes[nz].min()}/{group_sizes.max()}")
+    # the combine of the GPU's own y is exact arithmetic (f32 sum in slot order, one bf16 rounding)
+    toks = [0, 1, M - 1] + list(rng.integers(0, M, 5))
+    want_out = O.combine(yn, weights, inv_perm)[toks]
+    assert np.array_equal(H.bf16_to_np(out)[toks], want_out)
