@@ -329,3 +329,16 @@ def test_swiglu_closed_form():
     v = np.linspace(-10, 10, 1001)
     assert np.allclose(O.silu(v), v * (1 / (1 + np.exp(-v))))
     assert O.silu(np.float64(0)) == 0
+
+
+# ---------------------------------------------------------------- frozen fixture
+
+def test_oracle_matches_committed_fixture_for_config1():
+    """tests/golden/config1_oracle.npz (written by tests/golden/make_fixtures.py) freezes the oracle's results for
+    BASELINE config 1; the GPU tests compare against the live oracle, this keeps the oracle itself from drifting."""
+    import os
+    from tests.golden import make_fixtures
+    want = np.load(os.path.join(os.path.dirname(make_fixtures.__file__), "config1_oracle.npz"))
+    got = make_fixtures.build()
+    for name in want.files:
+        assert np.array_equal(want[name], got[name]), name
