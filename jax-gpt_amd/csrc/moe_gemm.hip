@@ -16,14 +16,17 @@
 // ONE activation row: one activation scale per lane per fragment, not four.
 //
 // Data movement.  A workgroup (8 waves, two per SIMD) owns a work item =
-// (expert, <= 128 activation rows, 256 weight rows) and walks K in steps of 128
-// through a ring of three LDS stages.  Tiles are copied global -> LDS by
-// global_load_lds (no registers in between), two steps ahead of the MFMAs.
-// In MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of the
+// (expert, <= BM activation rows, 256 weight rows) and walks K in steps of 128
+// through a ring of LDS stages.  Tiles are copied global -> LDS by
+// global_load_lds (no registers in between) ahead of their use.  In
+// MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of the
 // same output columns, so silu(g)*u is lane-local and the 1x128 amax stays
 // inside the workgroup.  Waves form a 4 x 2 grid: wave (wi, xj) owns weight rows
 // {32wi..32wi+31} of each half (GATEUP) or {64wi..64wi+63} (DOWN) against
-// activation rows [64 xj, 64 xj + 64): 4x4 MFMA tiles, 64 accumulator registers.
+// activation rows [BM/2 xj, +BM/2).  Two tile heights are built:
+//   BM = 128: wave tile 64 x 64, three stages of 48.5 KB (copies two steps ahead);
+//   BM = 256: wave tile 64 x 128, two stages of 65 KB (copies one, twice as long,
+//             step ahead); half the weight traffic, LDS reads and barriers per MFMA.
 //
 // Work items are listed on the device by build_items_kernel (no host read-back
 // of group sizes) in [expert][column block][row tile] order and dealt to the 8
@@ -38,16 +41,11 @@
 namespace {
 
 constexpr int BW = 256;       // weight rows per work item
-constexpr int BM = 128;       // activation rows per work item
 constexpr int BK = 128;       // K step = scale block
 constexpr int NWAVES = 8;
 constexpr int NT = 64 * NWAVES;
 constexpr int MODE_GATEUP = 0;
 constexpr int MODE_DOWN = 1;
-
-#ifndef MOE_VAR
-#define MOE_VAR 0   // development switch: bit 0 = no scale FMA, bit 1 = no copies in the loop
-#endif
 
 struct WorkHeader {
   int n_items;
@@ -109,7 +107,7 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
 
 // ---- main kernel ---------------------------------------------------------
 //
-// LDS stage = [weight tile 256 x 128 B][activation tile 128 x 128 B][128 activation scales].
+// LDS stage = [weight tile 256 x 128 B][activation tile BM x 128 B][BM activation scales].
 // Tiles are row-major with 128-byte rows; the 16-byte chunk c of row r sits at chunk position
 // c ^ ((r >> 1) & 7).  A fragment lane (row fr = lane % 16, quarter fq = lane / 16) feeds the
 // MFMA with K bytes [16 fq, +16) and [64 + 16 fq, +16) of its row -- the same choice for both
@@ -119,14 +117,26 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
 // consecutive tile rows; the swizzle is applied by choosing which 16-byte piece of the row
 // each lane fetches.  No asynchronous load ever targets a register.
 
-constexpr int NSTAGE = 3;
-constexpr int W_TILE_BYTES = BW * BK;              // 32 KB
-constexpr int X_TILE_BYTES = BM * BK;              // 16 KB
-constexpr int STAGE_X_OFF = W_TILE_BYTES;
-constexpr int STAGE_S_OFF = W_TILE_BYTES + X_TILE_BYTES;
-constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4;  // 49664
-constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;    // 148992
-constexpr int VM_PER_STEP = 7;                     // per wave per K step: 4 weight + 2 activation + 1 scale copy
+constexpr int MAX_KB = 256;   // K <= 32768
+constexpr int W_TILE_BYTES = BW * BK;   // 32 KB
+
+template <int XW>   // XW = 1: BM = 128, XW = 2: BM = 256
+struct Cfg {
+  static constexpr int BM = 128 * XW;
+  static constexpr int XF = 4 * XW;                            // activation fragments per wave
+  static constexpr int NSTAGE = XW == 1 ? 3 : 2;
+  static constexpr int PRE = NSTAGE - 1;                       // copies run PRE steps ahead
+  static constexpr int X_TILE_BYTES = BM * BK;
+  static constexpr int STAGE_X_OFF = W_TILE_BYTES;
+  static constexpr int STAGE_S_OFF = W_TILE_BYTES + X_TILE_BYTES;
+  static constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4;
+  static constexpr int WSCALE_OFF = NSTAGE * STAGE_BYTES;      // [2][MAX_KB] weight block scales of the work item
+  static constexpr int RING_BYTES = WSCALE_OFF + 2 * MAX_KB * 4;
+  static constexpr int EPI_BYTES = BM * 512;                   // bf16 staging of MODE_DOWN (<= RING_BYTES)
+  static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // 151040 / 133120
+  static constexpr int X_DMA = 2 * XW;                         // 1 KB activation row groups per wave per step
+  static constexpr int VM_PER_STEP = 4 + X_DMA + 1;            // + 4 weight row groups + 1 scale copy
+};
 
 // epilogue staging tile: 128-byte rows, chunk c of row r at position c ^ (r & 7)
 __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 4); }
@@ -134,21 +144,22 @@ __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chu
 // The copies are inline assembly on purpose: when the compiler knows that an instruction writes LDS from
 // memory it makes every later LDS read wait for ALL outstanding memory operations, which would empty the
 // prefetch queue at every K step.  Completion is tracked by hand instead (wait_vm + barrier); these are the
-// only vector-memory operations inside the K loop.  The LDS destination of lane l is m0 + l * size.
-__device__ __forceinline__ void dma16(const uint8_t* g, uint8_t* l) {
+// only vector-memory operations inside the K loop.  The LDS destination of lane l is m0 + l * size; the
+// source address is a uniform 64-bit base (scalar registers) + a per-lane 32-bit byte offset.
+__device__ __forceinline__ void dma16(const uint8_t* base, unsigned off, uint8_t* l) {
   const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
 }
-__device__ __forceinline__ void dma4(const float* g, uint8_t* l) {
+__device__ __forceinline__ void dma4(const uint8_t* base, unsigned off, uint8_t* l) {
   const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(m0v), "v"(g) : "memory", "m0");
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void wait_vm() {
   static_assert(N >= 0 && N < 64, "vmcnt range");
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));   // vmcnt = N, other counters untouched
 }
 
-template <int MODE>
+template <int MODE, int XW>
 __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0,   // gate (GATEUP) or down (DOWN)
@@ -156,6 +167,8 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const WorkHeader* __restrict__ hdr, const WorkItem* __restrict__ items,
     int K, int N,                                                    // contraction length; weight rows per matrix
     void* __restrict__ out, float* __restrict__ out_scale) {
+  using C = Cfg<XW>;
+  constexpr int BM = C::BM, XF = C::XF, HALF = BM / 2;
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // deal contiguous item ranges to the 8 XCDs (workgroup ids are issued round-robin over XCDs)
@@ -174,63 +187,67 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
   const int e = item.expert;
   const int wrow0 = MODE == MODE_GATEUP ? item.col_block * 128 : item.col_block * 256;
 
-  // ---- copy sources.  Wave w fills 1 KB row groups [4w, 4w+4) of the weight tile, [2w, 2w+2) of the
-  // activation tile and scale slots [16w, 16w+16).
+  // ---- copy sources.  Wave w fills 1 KB row groups [4w, 4w+4) of the weight tile, [X_DMA w, +X_DMA) of the
+  // activation tile and BM/8 scale slots.
   const int drow = lane >> 3, dchunk = lane & 7;
-  const uint8_t* wsrc[4];
+  // the weight rows of one wave all come from one matrix: waves 0-3 copy gate rows, 4-7 up rows
+  const uint8_t* wmat = (MODE == MODE_GATEUP && wave >= 4 ? w1 : w0) + (size_t)e * N * K;   // uniform
+  unsigned woff[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r = (wave * 4 + i) * 8 + drow;                   // row within the 256-row weight tile
     const int piece = dchunk ^ ((r >> 1) & 7);
-    const uint8_t* base;
-    int grow;
-    if (MODE == MODE_GATEUP) {
-      base = r < 128 ? w0 : w1;
-      grow = wrow0 + (r & 127);
-    } else {
-      base = w0;
-      grow = min(wrow0 + r, N - 1);
-    }
-    wsrc[i] = base + ((size_t)e * N + grow) * K + piece * 16;
+    const int grow = MODE == MODE_GATEUP ? wrow0 + (r & 127) : min(wrow0 + r, N - 1);
+    woff[i] = (unsigned)grow * (unsigned)K + piece * 16;       // < N*K <= 4 GB (checked by the launcher)
   }
-  const uint8_t* xsrc[2];
+  unsigned xoff[C::X_DMA];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int r = (wave * 2 + i) * 8 + drow;                   // row within the activation tile
+  for (int i = 0; i < C::X_DMA; ++i) {
+    const int r = (wave * C::X_DMA + i) * 8 + drow;            // row within the activation tile
     const int piece = dchunk ^ ((r >> 1) & 7);
     int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
-    xsrc[i] = xq + (size_t)g * K + piece * 16;
+    xoff[i] = (unsigned)g * (unsigned)K + piece * 16;          // < rows*K <= 4 GB (checked by the launcher)
   }
-  // scale slot 64 h + fr * 4 + j holds the scale of tile row 64 h + 16 j + fr: a lane reads its 4 scales as 16 bytes
-  const float* ssrc;
+  // scale slot HALF h + fr * XF + j holds the scale of tile row HALF h + 16 j + fr: a lane reads its XF scales
+  // as XF * 4 contiguous bytes.  Wave w copies slots [BM/8 w, +BM/8).
+  unsigned soff;
   {
-    const int p = wave * 16 + (lane & 15);
-    const int q = p & 63;
-    const int r = (p & 64) + 16 * (q & 3) + (q >> 2);
+    const int p = wave * (BM / 8) + (lane & (BM / 8 - 1));
+    const int q = p % HALF;
+    const int r = (p / HALF) * HALF + 16 * (q % XF) + q / XF;
     int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
-    ssrc = sx + (size_t)g * KB;
+    soff = (unsigned)g * (unsigned)KB * 4u;
   }
   auto issue = [&](int kb) {   // VM_PER_STEP operations
-    uint8_t* st = lds + (kb % NSTAGE) * STAGE_BYTES;
+    uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
+    const uint8_t* wk = wmat + (size_t)kb * BK;
+    const uint8_t* xk = xq + (size_t)kb * BK;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma16(wsrc[i] + (size_t)kb * BK, st + (wave * 4 + i) * 1024);
+    for (int i = 0; i < 4; ++i) dma16(wk, woff[i], st + (wave * 4 + i) * 1024);
 #pragma unroll
-    for (int i = 0; i < 2; ++i) dma16(xsrc[i] + (size_t)kb * BK, st + STAGE_X_OFF + (wave * 2 + i) * 1024);
-    if (lane < 16) dma4(ssrc + kb, st + STAGE_S_OFF + wave * 64);
+    for (int i = 0; i < C::X_DMA; ++i) dma16(xk, xoff[i], st + C::STAGE_X_OFF + (wave * C::X_DMA + i) * 1024);
+    if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4);
   };
+  // start the pipeline before anything else waits on memory
+  issue(0);
+  if (C::PRE > 1 && KB > 1) issue(1);
 
-  // weight scales of this wave's rows
-  const float* swp0;
-  const float* swp1 = nullptr;
-  if (MODE == MODE_GATEUP) {
-    swp0 = sw0 + ((size_t)e * (N / 128) + item.col_block) * KB;
-    swp1 = sw1 + ((size_t)e * (N / 128) + item.col_block) * KB;
-  } else {
-    const int nb = min(item.col_block * 2 + (wi >> 1), N / 128 - 1);
-    swp0 = sw0 + ((size_t)e * (N / 128) + nb) * KB;
+  // Weight block scales of this work item go to LDS once: [0][kb] = gate (or the first 128 down rows), [1][kb] =
+  // up (or the second 128 down rows).  Scalar loads inside the K loop would force every LDS wait to
+  // lgkmcnt(0) (they share that counter and return out of order).
+  float* wscale = (float*)(lds + C::WSCALE_OFF);
+  for (int i = tid; i < 2 * KB; i += NT) {
+    const int h = i >= KB, kk = h ? i - KB : i;
+    float v;
+    if (MODE == MODE_GATEUP) v = (h ? sw1 : sw0)[((size_t)e * (N / 128) + item.col_block) * KB + kk];
+    else v = sw0[((size_t)e * (N / 128) + min(item.col_block * 2 + h, N / 128 - 1)) * KB + kk];
+    wscale[h * MAX_KB + kk] = v;
   }
+  const float* ws0 = wscale + (MODE == MODE_GATEUP ? 0 : (wi >> 1) * MAX_KB);
+  const float* ws1 = wscale + MAX_KB;   // GATEUP only
+  __syncthreads();   // (the compiler waits here for the scale loads, and with them for the copies issued above)
 
   const int lane_off0 = fr * BK + ((fq ^ (fr >> 1)) << 4);         // K bytes [16 fq, +16)
   const int lane_off1 = fr * BK + (((fq + 4) ^ (fr >> 1)) << 4);   // K bytes [64 + 16 fq, +16)
@@ -239,86 +256,75 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
   for (int f = 0; f < 4; ++f)
     wfrag_off[f] = (MODE == MODE_GATEUP ? ((f >> 1) * 128 + wi * 32 + (f & 1) * 16) : (wi * 64 + f * 16)) * BK;
   // activation fragments past the item's last row are never multiplied (uniform per wave)
-  const int jmax = min(4, max(0, (item.row_count - xj * 64 + 15) >> 4));
+  const int jmax = min(XF, max(0, (item.row_count - xj * HALF + 15) >> 4));
 
-  v4f acc[4][4];
+  v4f acc[4][XF];
 #pragma unroll
   for (int f = 0; f < 4; ++f)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[f][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < XF; ++j) acc[f][j] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  issue(0);
-  if (KB > 1) issue(1);
-  float s0n = swp0[0], s1n = MODE == MODE_GATEUP ? swp1[0] : 0.f;
+  auto read_frag = [&](const uint8_t* base) {
+    const v4i lo = *(const v4i*)(base + lane_off0);
+    const v4i hi = *(const v4i*)(base + lane_off1);
+    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
 
   for (int kb = 0; kb < KB; ++kb) {
-    // stage kb has landed once only the next step's copies are still outstanding
-    if (MOE_VAR & 2) {
-    } else if (kb + 1 < KB) {
-      wait_vm<VM_PER_STEP>();
-    } else {
-      wait_vm<0>();
-    }
+    // stage kb has landed once only the younger steps' copies are outstanding
+    if (C::PRE > 1 && kb + 1 < KB) wait_vm<C::VM_PER_STEP>();
+    else wait_vm<0>();
     __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; stage (kb-1) % NSTAGE is free again
-    if (!(MOE_VAR & 2) && kb + 2 < KB) issue(kb + 2);
+    if (kb + C::PRE < KB) issue(kb + C::PRE);
 
-    const uint8_t* st = lds + (kb % NSTAGE) * STAGE_BYTES;
-    const float s0 = s0n, s1 = MODE == MODE_GATEUP ? s1n : s0n;
-    if (kb + 1 < KB) {   // next step's weight scales, one step early
-      s0n = swp0[kb + 1];
-      if (MODE == MODE_GATEUP) s1n = swp1[kb + 1];
-    }
-    auto read_frag = [&](const uint8_t* base) {
-      const v4i lo = *(const v4i*)(base + lane_off0);
-      const v4i hi = *(const v4i*)(base + lane_off1);
-      return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-    };
-    const uint8_t* xt = st + STAGE_X_OFF + xj * 64 * BK;
-    v8i wf[4], xf[4];
+    const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
+    const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
+    const uint8_t* xt = st + C::STAGE_X_OFF + xj * HALF * BK;
+    v8i wf[4];
 #pragma unroll
     for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
+    float sxv[XF];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) xf[j] = read_frag(xt + j * 16 * BK);
-    float sc0[4], sc1[4];
-    {
-      const v4f a = *(const v4f*)(st + STAGE_S_OFF + xj * 256 + fr * 16);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        sc0[j] = a[j] * s0;
-        sc1[j] = a[j] * s1;
-      }
+    for (int j = 0; j < XF; j += 4) {
+      const v4f a = *(const v4f*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + j * 4);
+      sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
     }
     // one uniform branch per K step: the common full tile runs a branch-free schedule
     auto mma = [&](auto full) {
       constexpr bool FULL = decltype(full)::value;
+      constexpr int XA = XW == 1 ? 2 : 1;   // activation fragments are read XA MFMA groups ahead (registers allow 1 at BM = 256)
+      v8i xf[XA + 1];
       v4f p[2][4];
 #pragma unroll
-      for (int j = 0; j <= 4; ++j) {
-        if (j < 4 && (FULL || j < jmax)) {
+      for (int j = 0; j < XA; ++j) xf[j] = read_frag(xt + j * 16 * BK);
+#pragma unroll
+      for (int j = 0; j <= XF; ++j) {
+        if (j + XA < XF) xf[(j + XA) % (XA + 1)] = read_frag(xt + (j + XA) * 16 * BK);
+        if (j < XF && (FULL || j < jmax)) {
 #pragma unroll
           for (int f = 0; f < 4; ++f)
-            if (MOE_VAR & 1) acc[f][j] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf[j], acc[f][j], 0, 0, 0, 0, 0, 0);
-            else p[j & 1][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf[j], (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+            p[j & 1][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf[j % (XA + 1)], (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
         }
-        if (!(MOE_VAR & 1) && j > 0 && (FULL || j - 1 < jmax)) {
+        if (j > 0 && (FULL || j - 1 < jmax)) {
           const int jj = j - 1;
+          const float c0 = sxv[jj] * s0, c1 = sxv[jj] * s1;
 #pragma unroll
-          for (int f = 0; f < 4; ++f)
-            acc[f][jj] += p[jj & 1][f] * ((MODE == MODE_GATEUP && f >= 2) ? sc1[jj] : sc0[jj]);
+          for (int f = 0; f < 4; ++f) acc[f][jj] += p[jj & 1][f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
         }
       }
     };
-    if (jmax == 4) mma(std::true_type{});
+    // (at BM = 256 two copies of the schedule do not fit the register file next to 128 accumulators)
+    if (XW == 1 && jmax == XF) mma(std::true_type{});
     else mma(std::false_type{});
   }
   __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
 
-  // ---- epilogue.  Lane holds, for fragment (f, j): tile row xj*64 + j*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
+  // ---- epilogue.  Lane holds, for fragment (f, j): tile row xj*HALF + j*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
   if (MODE == MODE_GATEUP) {
-    float* amax_s = (float*)lds;                       // [4 weight-wave groups][128 rows]
-    uint8_t* tile = lds + 4 * BM * sizeof(float);      // [128 rows][128 B], swizzled
+    float* amax_s = (float*)lds;                       // [4 weight-wave groups][BM rows]
+    uint8_t* tile = lds + 4 * BM * sizeof(float);      // [BM rows][128 B], swizzled
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < XF; ++j) {
       float m = 0.f;
 #pragma unroll
       for (int f = 0; f < 2; ++f)
@@ -331,14 +337,14 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
         }
       m = fmaxf(m, __shfl_xor(m, 16, MOE_WAVE));
       m = fmaxf(m, __shfl_xor(m, 32, MOE_WAVE));
-      if (fq == 0) amax_s[wi * BM + xj * 64 + j * 16 + fr] = m;
+      if (fq == 0) amax_s[wi * BM + xj * HALF + j * 16 + fr] = m;
     }
     __syncthreads();
     const int I = N;
     uint8_t* hq = (uint8_t*)out;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int xr = xj * 64 + j * 16 + fr;
+    for (int j = 0; j < XF; ++j) {
+      const int xr = xj * HALF + j * 16 + fr;
       float m = fmaxf(fmaxf(amax_s[xr], amax_s[BM + xr]), fmaxf(amax_s[2 * BM + xr], amax_s[3 * BM + xr]));
       float scale, scale_inv;
       fp8_scales(m, scale, scale_inv);
@@ -354,7 +360,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     __syncthreads();
     const int ld_chunk = tid & 7, ld_row = tid >> 3;   // 64 rows per pass
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < BM / 64; ++i) {
       const int r = ld_row + 64 * i;
       if (r < item.row_count) {
         v4i v = *(const v4i*)(tile + swz(r, ld_chunk));
@@ -362,11 +368,11 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
       }
     }
   } else {
-    // bf16 tile [128 rows][256 cols] = 512 B per row, 32 chunks of 16 B, swizzled with (row & 7)
+    // bf16 tile [BM rows][256 cols] = 512 B per row, 32 chunks of 16 B, swizzled with (row & 7)
     uint8_t* tile = lds;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int xr = xj * 64 + j * 16 + fr;
+    for (int j = 0; j < XF; ++j) {
+      const int xr = xj * HALF + j * 16 + fr;
 #pragma unroll
       for (int f = 0; f < 4; ++f) {
         const int col = wi * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
@@ -382,7 +388,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const int c32 = tid & 31, r16 = tid >> 5;          // 16 rows per pass
     const int ncols = min(256, N - wrow0);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < BM / 16; ++i) {
       const int r = r16 + 16 * i;
       if (r < item.row_count && c32 * 8 < ncols) {
         v4i v = *(const v4i*)(tile + r * 512 + ((c32 ^ (r & 7)) << 4));
@@ -392,9 +398,41 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
   }
 }
 
-int max_items_for(int R, int E, int n_col_blocks) {
-  long long tiles = (long long)(R + BM - 1) / BM + (E < R ? E : R);
+int max_items_for(int R, int E, int n_col_blocks, int bm) {
+  long long tiles = (long long)(R + bm - 1) / bm + (E < R ? E : R);
   return (int)(tiles * n_col_blocks);
+}
+
+template <int MODE, int XW>
+int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
+               const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
+               void* out, float* out_scale, void* ws, hipStream_t s) {
+  using C = Cfg<XW>;
+  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
+  const int max_items = max_items_for(R, E, ncb, C::BM);
+  WorkHeader* hdr = (WorkHeader*)ws;
+  WorkItem* items = (WorkItem*)((char*)ws + sizeof(WorkHeader));
+  hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, ncb, C::BM, max_items, hdr, items);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t err = hipFuncSetAttribute((const void*)grouped_gemm_kernel<MODE, XW>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+    if (err != hipSuccess) return moe_check_hip(err, "gemm: raising the dynamic LDS limit");
+    attr_set = true;
+  }
+  const int grid = ((max_items + 7) / 8) * 8;
+  hipLaunchKernelGGL((grouped_gemm_kernel<MODE, XW>), dim3(grid), dim3(NT), C::LDS_BYTES, s, xq, sx, row_ids, w0, sw0,
+                     w1, sw1, hdr, items, K, N, out, out_scale);
+  return moe_check_hip(hipGetLastError(), "gemm launch");
+}
+
+// MOE_GEMM_BM=128|256 in the environment pins the tile height for experiments; default: by shape
+int forced_xw() {
+  static int v = [] {
+    const char* e = getenv("MOE_GEMM_BM");
+    return e ? atoi(e) : 0;
+  }();
+  return v == 128 ? 1 : v == 256 ? 2 : 0;
 }
 
 template <int MODE>
@@ -403,31 +441,23 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
            void* out, float* out_scale, void* ws, size_t ws_bytes, hipStream_t s) {
   const size_t need = moe_gemm_workspace_bytes(R, E, N);
   MOE_REQUIRE(ws_bytes >= need, MOE_ERR_WORKSPACE_TOO_SMALL, "gemm: workspace %zu < %zu", ws_bytes, need);
+  MOE_REQUIRE(K <= MAX_KB * BK, MOE_ERR_BAD_SHAPE, "gemm: contraction length %d exceeds %d", K, MAX_KB * BK);
+  MOE_REQUIRE((long long)N * K <= (1ll << 32) && (long long)R * K <= (1ll << 32), MOE_ERR_BAD_SHAPE,
+              "gemm: one expert matrix and the activation array must each stay within 4 GB (N=%d K=%d R=%d)", N, K, R);
   if (R == 0) return MOE_OK;
-  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
-  const int max_items = max_items_for(R, E, ncb);
-  WorkHeader* hdr = (WorkHeader*)ws;
-  WorkItem* items = (WorkItem*)((char*)ws + sizeof(WorkHeader));
-  hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, ncb, BM, max_items, hdr, items);
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t err = hipFuncSetAttribute((const void*)grouped_gemm_kernel<MODE>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
-    if (err != hipSuccess) return moe_check_hip(err, "gemm: raising the dynamic LDS limit");
-    attr_set = true;
-  }
-  const int grid = ((max_items + 7) / 8) * 8;
-  hipLaunchKernelGGL(grouped_gemm_kernel<MODE>, dim3(grid), dim3(NT), LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1, sw1,
-                     hdr, items, K, N, out, out_scale);
-  return moe_check_hip(hipGetLastError(), "gemm launch");
+  // 256-row tiles once the average expert has more than 128 rows, 128-row tiles otherwise
+  const int xw = forced_xw() ? forced_xw() : ((long long)R > 128ll * E ? 2 : 1);
+  if (xw == 2)
+    return launch_cfg<MODE, 2>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws, s);
+  return launch_cfg<MODE, 1>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws, s);
 }
 
 }  // namespace
 
 extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
-  // enough for either GEMM: column blocks of 128 bound both cases
+  // enough for either GEMM and either tile height: column blocks of 128 and 128-row tiles bound every case
   int ncb = (N_out + 127) / 128;
-  return sizeof(WorkHeader) + (size_t)max_items_for(R, E, ncb) * sizeof(WorkItem) + 256;
+  return sizeof(WorkHeader) + (size_t)max_items_for(R, E, ncb, 128) * sizeof(WorkItem) + 256;
 }
 
 extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
