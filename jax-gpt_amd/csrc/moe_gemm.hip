@@ -22,16 +22,22 @@
 // MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of the
 // same output columns, so silu(g)*u is lane-local and the 1x128 amax stays
 // inside the workgroup.  Waves form a 4 x 2 grid: wave (wi, xj) owns weight rows
-// {32wi..32wi+31} of each half (GATEUP) or {64wi..64wi+63} (DOWN) against
-// activation rows [BM/2 xj, +BM/2).  Two tile heights are built:
+// {32wi..32wi+31} of each half (GATEUP) or {64wi..64wi+63} (DOWN) against the
+// 16-row activation fragments 2j + xj (alternating between the two wave sets, so
+// a short tile still splits evenly).  Two tile heights are built:
 //   BM = 128: wave tile 64 x 64, three stages of 48.5 KB (copies two steps ahead);
 //   BM = 256: wave tile 64 x 128, two stages of 65 KB (copies one, twice as long,
 //             step ahead); half the weight traffic, LDS reads and barriers per MFMA.
 //
+// The copies of a step are issued a few at a time between MFMA groups, not in
+// one burst, and the two waves of each SIMD run out of phase (see the K loop).
+//
 // Work items are listed on the device by build_items_kernel (no host read-back
 // of group sizes) in [expert][column block][row tile] order and dealt to the 8
 // XCDs in contiguous ranges, so the row tiles and column blocks that share a
-// weight slab or an activation tile run together under one L2.
+// weight slab or an activation tile run together under one L2.  An expert's
+// rows are cut into tiles of equal height, so that the tiles sharing a weight
+// slab advance at the same pace.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -57,7 +63,13 @@ struct WorkItem {
 
 // ---- work list -----------------------------------------------------------
 
-// One workgroup.  tiles[e] = ceil(rows_e / bm); item order [expert][col_block][row tile].
+// One workgroup.  An expert with rows_e rows gets ceil(rows_e / bm) row tiles of equal height (a multiple of 16,
+// the last one shorter): tiles that share a weight slab then take the same time per K step and walk it together,
+// so the second reader finds it in L2.  Item order [expert][col_block][row tile].
+__device__ __forceinline__ int tile_rows(int rows, int bm) {
+  const int t = (rows + bm - 1) / bm;
+  return t <= 1 ? bm : (((rows + t - 1) / t + 15) & ~15);
+}
 __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __restrict__ group_offsets, int E,
                                                           int n_col_blocks, int bm, int max_items,
                                                           WorkHeader* __restrict__ hdr, WorkItem* __restrict__ items) {
@@ -67,7 +79,11 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
   const int lane = e & 63, wv = e >> 6;
   int rows = 0;
   if (e < E) rows = group_offsets[e + 1] - group_offsets[e];
-  int tiles = rows > 0 ? (rows + bm - 1) / bm : 0;
+  int tiles = 0;
+  if (rows > 0) {
+    const int tr = tile_rows(rows, bm);
+    tiles = (rows + tr - 1) / tr;
+  }
   int incl = tiles;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -96,10 +112,11 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
     const int local = it - tile_prefix[x] * n_col_blocks;
     const int cb = local / tiles_x, rt = local % tiles_x;
     const int start = group_offsets[x], rows_x = group_offsets[x + 1] - start;
+    const int tr = tile_rows(rows_x, bm);
     WorkItem w;
     w.expert = x;
-    w.row_start = start + rt * bm;
-    w.row_count = min(bm, rows_x - rt * bm);
+    w.row_start = start + rt * tr;
+    w.row_count = min(tr, rows_x - rt * tr);
     w.col_block = cb;
     items[it] = w;
   }
@@ -136,6 +153,32 @@ struct Cfg {
   static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // 151040 / 133120
   static constexpr int X_DMA = 2 * XW;                         // 1 KB activation row groups per wave per step
   static constexpr int VM_PER_STEP = 4 + X_DMA + 1;            // + 4 weight row groups + 1 scale copy
+  // MFMA groups by which wave set 1 trails wave set 0 (build-time tuning knobs; measured best: half a step at
+  // BM = 128, one group at BM = 256 where registers are short)
+#ifndef MOE_ROT1
+#define MOE_ROT1 2
+#endif
+#ifndef MOE_ROT2
+#define MOE_ROT2 1
+#endif
+  static constexpr int ROT = XW == 1 ? MOE_ROT1 : MOE_ROT2;
+};
+
+// Sched<XW>::first(j) = index of the first copy operation issued after MFMA group j (first(XF) = VM_PER_STEP).
+// MOE_SCHED (build-time tuning knob): 0 = all copies at the start of the step, 1 = spread evenly, 2 / 3 = spread
+// over the first half / three quarters of the step (3 measured best).
+#ifndef MOE_SCHED
+#define MOE_SCHED 3
+#endif
+template <int XW> struct Sched {
+  static constexpr int first(int j) {
+    constexpr int n = Cfg<XW>::VM_PER_STEP, g = Cfg<XW>::XF;
+    if (j >= g) return n;
+    if (MOE_SCHED == 1) return (n * j) / g;                    // even
+    if (MOE_SCHED == 2) { int h = g / 2; return j >= h ? n : (n * j) / h; }   // all in the first half of the step
+    if (MOE_SCHED == 3) { int h = (3 * g) / 4; return j >= h ? n : (n * j) / h; }
+    return j == 0 ? 0 : n;
+  }
 };
 
 // epilogue staging tile: 128-byte rows, chunk c of row r at position c ^ (r & 7)
@@ -154,6 +197,7 @@ __device__ __forceinline__ void dma4(const uint8_t* base, unsigned off, uint8_t*
   const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
 }
+__device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(0xC07F); }   // lgkmcnt = 0, other counters untouched
 template <int N> __device__ __forceinline__ void wait_vm() {
   static_assert(N >= 0 && N < 64, "vmcnt range");
   __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));   // vmcnt = N, other counters untouched
@@ -209,26 +253,28 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     if (row_ids) g = row_ids[g];
     xoff[i] = (unsigned)g * (unsigned)K + piece * 16;          // < rows*K <= 4 GB (checked by the launcher)
   }
-  // scale slot HALF h + fr * XF + j holds the scale of tile row HALF h + 16 j + fr: a lane reads its XF scales
-  // as XF * 4 contiguous bytes.  Wave w copies slots [BM/8 w, +BM/8).
+  // 16-row fragment 2j + h of the tile belongs to wave set h (its j-th), so a short tile still splits evenly between
+  // the sets.  Scale slot HALF h + fr * XF + j holds the scale of tile row 16 (2j + h) + fr: a lane reads its XF
+  // scales as XF * 4 contiguous bytes.  Wave w copies slots [BM/8 w, +BM/8).
   unsigned soff;
   {
     const int p = wave * (BM / 8) + (lane & (BM / 8 - 1));
     const int q = p % HALF;
-    const int r = (p / HALF) * HALF + 16 * (q % XF) + q / XF;
+    const int r = 16 * (2 * (q % XF) + p / HALF) + q / XF;
     int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
     soff = (unsigned)g * (unsigned)KB * 4u;
   }
-  auto issue = [&](int kb) {   // VM_PER_STEP operations
+  // copy operation i (0 <= i < VM_PER_STEP) of K step kb
+  auto issue_op = [&](int kb, int i) {
     uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
-    const uint8_t* wk = wmat + (size_t)kb * BK;
-    const uint8_t* xk = xq + (size_t)kb * BK;
+    if (i < 4) dma16(wmat + (size_t)kb * BK, woff[i], st + (wave * 4 + i) * 1024);
+    else if (i < 4 + C::X_DMA) dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + (wave * C::X_DMA + i - 4) * 1024);
+    else if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4);
+  };
+  auto issue = [&](int kb) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) dma16(wk, woff[i], st + (wave * 4 + i) * 1024);
-#pragma unroll
-    for (int i = 0; i < C::X_DMA; ++i) dma16(xk, xoff[i], st + C::STAGE_X_OFF + (wave * C::X_DMA + i) * 1024);
-    if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4);
+    for (int i = 0; i < C::VM_PER_STEP; ++i) issue_op(kb, i);
   };
   // start the pipeline before anything else waits on memory
   issue(0);
@@ -256,7 +302,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
   for (int f = 0; f < 4; ++f)
     wfrag_off[f] = (MODE == MODE_GATEUP ? ((f >> 1) * 128 + wi * 32 + (f & 1) * 16) : (wi * 64 + f * 16)) * BK;
   // activation fragments past the item's last row are never multiplied (uniform per wave)
-  const int jmax = min(XF, max(0, (item.row_count - xj * HALF + 15) >> 4));
+  const int jmax = (((item.row_count + 15) >> 4) + 1 - xj) >> 1;
 
   v4f acc[4][XF];
 #pragma unroll
@@ -270,56 +316,109 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
   };
 
-  for (int kb = 0; kb < KB; ++kb) {
-    // stage kb has landed once only the younger steps' copies are outstanding
-    if (C::PRE > 1 && kb + 1 < KB) wait_vm<C::VM_PER_STEP>();
-    else wait_vm<0>();
-    __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; stage (kb-1) % NSTAGE is free again
-    if (kb + C::PRE < KB) issue(kb + C::PRE);
-
-    const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
-    const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
-    const uint8_t* xt = st + C::STAGE_X_OFF + xj * HALF * BK;
-    v8i wf[4];
+  // One K step = XF MFMA groups (one activation fragment against the wave's four weight fragments).  The two
+  // waves of a SIMD belong to different wave sets (xj = 0 / 1); set 1 runs ROT groups behind set 0, carrying the
+  // last ROT activation fragments of a step in registers across the barrier, so that after a barrier one wave of
+  // each SIMD still has matrix work in registers while the other waits for its first fragments from LDS.
+  auto run = [&](auto rot_c, auto full_c) {
+    constexpr int ROT = decltype(rot_c)::value;
+    constexpr bool FULL = decltype(full_c)::value;
+    constexpr int NG = XF - ROT;          // groups of the current step done before the next barrier
+    constexpr int XA = XW == 1 ? 2 : 1;   // activation fragments are read XA groups ahead
+    constexpr int NH = ROT > 0 ? ROT : 1;
+    v8i wf[4], held[NH];
+    float hc0[NH], hc1[NH];
+    v4f p[2][4];
+    auto mm = [&](int pp, const v8i& x) {
 #pragma unroll
-    for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
-    float sxv[XF];
+      for (int f = 0; f < 4; ++f)
+        p[pp][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], x, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+    };
+    auto fm = [&](int pp, int jj, float c0, float c1) {
 #pragma unroll
-    for (int j = 0; j < XF; j += 4) {
-      const v4f a = *(const v4f*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + j * 4);
-      sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
-    }
-    // one uniform branch per K step: the common full tile runs a branch-free schedule
-    auto mma = [&](auto full) {
-      constexpr bool FULL = decltype(full)::value;
-      constexpr int XA = XW == 1 ? 2 : 1;   // activation fragments are read XA MFMA groups ahead (registers allow 1 at BM = 256)
-      v8i xf[XA + 1];
-      v4f p[2][4];
+      for (int f = 0; f < 4; ++f) acc[f][jj] += p[pp][f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
+    };
+    auto late = [&](bool more, int kb_next) {   // groups NG .. XF-1 of the previous step; the last FMA is left to the caller
 #pragma unroll
-      for (int j = 0; j < XA; ++j) xf[j] = read_frag(xt + j * 16 * BK);
+      for (int i = 0; i < ROT; ++i) {
+        const int j = NG + i;
+        if (FULL || j < jmax) mm(i & 1, held[i]);
+        if (more) {
 #pragma unroll
-      for (int j = 0; j <= XF; ++j) {
-        if (j + XA < XF) xf[(j + XA) % (XA + 1)] = read_frag(xt + (j + XA) * 16 * BK);
-        if (j < XF && (FULL || j < jmax)) {
-#pragma unroll
-          for (int f = 0; f < 4; ++f)
-            p[j & 1][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], xf[j % (XA + 1)], (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+          for (int o = Sched<XW>::first(i); o < Sched<XW>::first(i + 1); ++o) issue_op(kb_next, o);
         }
-        if (j > 0 && (FULL || j - 1 < jmax)) {
-          const int jj = j - 1;
-          const float c0 = sxv[jj] * s0, c1 = sxv[jj] * s1;
-#pragma unroll
-          for (int f = 0; f < 4; ++f) acc[f][jj] += p[jj & 1][f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
-        }
+        if (i > 0 && (FULL || j - 1 < jmax)) fm((i - 1) & 1, j - 1, hc0[i - 1], hc1[i - 1]);
       }
     };
-    // (at BM = 256 two copies of the schedule do not fit the register file next to 128 accumulators)
-    if (XW == 1 && jmax == XF) mma(std::true_type{});
-    else mma(std::false_type{});
+    for (int kb = 0; kb < KB; ++kb) {
+      // stage kb has landed once only the younger steps' copies are outstanding
+      if (C::PRE > 1 && kb + 1 < KB) wait_vm<C::VM_PER_STEP>();
+      else wait_vm<0>();
+      if (ROT > 0) wait_lgkm0();      // this wave's reads of stage kb-1 are done before anyone overwrites it
+      __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; stage (kb-1) % NSTAGE is free again
+      const bool more = kb + C::PRE < KB;   // uniform
+      if (ROT > 0) {
+        if (kb > 0) late(more, kb + C::PRE);
+        else if (more) {
+#pragma unroll
+          for (int o = 0; o < Sched<XW>::first(ROT); ++o) issue_op(kb + C::PRE, o);
+        }
+      }
+      const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
+      const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
+      const uint8_t* xt = st + C::STAGE_X_OFF + xj * 16 * BK;
+#pragma unroll
+      for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
+      float sxv[XF];
+#pragma unroll
+      for (int j = 0; j < XF; j += 4) {
+        const v4f a = *(const v4f*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + j * 4);
+        sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
+      }
+      v8i xf[XA + 1];
+#pragma unroll
+      for (int j = 0; j < XA; ++j) xf[j] = read_frag(xt + j * 32 * BK);
+      if (ROT > 0 && kb > 0 && (FULL || XF - 1 < jmax)) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
+#pragma unroll
+      for (int j = 0; j <= NG; ++j) {
+        if (j + XA < NG) xf[(j + XA) % (XA + 1)] = read_frag(xt + (j + XA) * 32 * BK);
+        if (j < NG && (FULL || j < jmax)) mm(j & 1, xf[j % (XA + 1)]);
+        // the copies for step kb + PRE are spread over the MFMA groups: issued in one burst they hold every wave
+        // at the memory pipeline's front door while the matrix cores idle
+        if (j < NG && more) {
+#pragma unroll
+          for (int o = Sched<XW>::first(ROT + j); o < Sched<XW>::first(ROT + j + 1); ++o) issue_op(kb + C::PRE, o);
+        }
+        if (ROT > 0 && j == 0) {
+#pragma unroll
+          for (int i = 0; i < ROT; ++i) {
+            held[i] = read_frag(xt + (NG + i) * 32 * BK);
+            hc0[i] = sxv[NG + i] * s0;
+            hc1[i] = sxv[NG + i] * s1;
+          }
+        }
+        if (j > 0 && (FULL || j - 1 < jmax)) fm((j - 1) & 1, j - 1, sxv[j - 1] * s0, sxv[j - 1] * s1);
+      }
+    }
+    if (ROT > 0) {
+      late(false, 0);
+      if (FULL || XF - 1 < jmax) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
+    }
+  };
+  // one uniform branch per work item: the common full tile runs a branch-free schedule
+  // (at BM = 256 two copies of the schedule do not fit the register file next to 128 accumulators)
+  constexpr int ROT = C::ROT;
+  const bool full = XW == 1 && jmax == XF;
+  if (ROT == 0 || xj == 0) {
+    if (full) run(std::integral_constant<int, 0>{}, std::true_type{});
+    else run(std::integral_constant<int, 0>{}, std::false_type{});
+  } else {
+    if (full) run(std::integral_constant<int, ROT>{}, std::true_type{});
+    else run(std::integral_constant<int, ROT>{}, std::false_type{});
   }
   __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
 
-  // ---- epilogue.  Lane holds, for fragment (f, j): tile row xj*HALF + j*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
+  // ---- epilogue.  Lane holds, for fragment (f, j): tile row (2j + xj)*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
   if (MODE == MODE_GATEUP) {
     float* amax_s = (float*)lds;                       // [4 weight-wave groups][BM rows]
     uint8_t* tile = lds + 4 * BM * sizeof(float);      // [BM rows][128 B], swizzled
@@ -337,14 +436,14 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
         }
       m = fmaxf(m, __shfl_xor(m, 16, MOE_WAVE));
       m = fmaxf(m, __shfl_xor(m, 32, MOE_WAVE));
-      if (fq == 0) amax_s[wi * BM + xj * HALF + j * 16 + fr] = m;
+      if (fq == 0) amax_s[wi * BM + (2 * j + xj) * 16 + fr] = m;
     }
     __syncthreads();
     const int I = N;
     uint8_t* hq = (uint8_t*)out;
 #pragma unroll
     for (int j = 0; j < XF; ++j) {
-      const int xr = xj * HALF + j * 16 + fr;
+      const int xr = (2 * j + xj) * 16 + fr;
       float m = fmaxf(fmaxf(amax_s[xr], amax_s[BM + xr]), fmaxf(amax_s[2 * BM + xr], amax_s[3 * BM + xr]));
       float scale, scale_inv;
       fp8_scales(m, scale, scale_inv);
@@ -372,7 +471,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     uint8_t* tile = lds;
 #pragma unroll
     for (int j = 0; j < XF; ++j) {
-      const int xr = xj * HALF + j * 16 + fr;
+      const int xr = (2 * j + xj) * 16 + fr;
 #pragma unroll
       for (int f = 0; f < 4; ++f) {
         const int col = wi * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
