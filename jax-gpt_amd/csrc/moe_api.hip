@@ -5,6 +5,8 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+
 #include "moe_common.h"
 
 static thread_local char g_err[512] = "";
@@ -34,6 +36,23 @@ __global__ void dense_offsets_kernel(int32_t* off, int M) {
   }
 }
 
+// One side stream per device, default priority, created on first use and kept for the life of the process.
+int side_stream(hipStream_t* out) {
+  static std::mutex mu;
+  static hipStream_t streams[64] = {};
+  int dev = 0;
+  int rc = moe_check_hip(hipGetDevice(&dev), "forward: hipGetDevice");
+  if (rc) return rc;
+  if (dev < 0 || dev >= 64) return moe_set_error(MOE_ERR_HIP, "forward: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!streams[dev]) {
+    if ((rc = moe_check_hip(hipStreamCreateWithFlags(&streams[dev], hipStreamNonBlocking), "forward: side stream")))
+      return rc;
+  }
+  *out = streams[dev];
+  return MOE_OK;
+}
+
 struct Carver {
   char* base;
   size_t used;
@@ -48,8 +67,8 @@ struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
   float *w, *sx, *sh, *shs;
   uint8_t *xq, *hq, *hsq;
-  void *y, *ys, *permute_ws, *gemm_ws;
-  size_t permute_ws_bytes, gemm_ws_bytes, total;
+  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_shared;
+  size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, total;
 };
 
 ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
@@ -65,10 +84,11 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
   b.dense_off = (int32_t*)c.take(8);
   b.permute_ws_bytes = moe_permute_workspace_bytes(M, k, E);
   b.permute_ws = c.take(b.permute_ws_bytes);
-  size_t g1 = moe_gemm_workspace_bytes((int)R, E, I > D ? I : D);
-  size_t g2 = SI ? moe_gemm_workspace_bytes(M, 1, SI > D ? SI : D) : 0;
-  b.gemm_ws_bytes = g1 > g2 ? g1 : g2;
+  b.gemm_ws_bytes = moe_gemm_workspace_bytes((int)R, E, I > D ? I : D);
   b.gemm_ws = c.take(b.gemm_ws_bytes);
+  // the shared expert runs beside the routed ones on its own stream: its launches need their own work lists
+  b.gemm_ws_shared_bytes = SI ? moe_gemm_workspace_bytes(M, 1, SI > D ? SI : D) : 0;
+  b.gemm_ws_shared = SI ? c.take(b.gemm_ws_shared_bytes) : nullptr;
   b.xq = (uint8_t*)c.take((size_t)M * D);
   b.sx = (float*)c.take((size_t)M * (D / 128) * 4);
   b.hq = (uint8_t*)c.take(R * I);
@@ -111,34 +131,67 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   int32_t* stid = a->out_sorted_token_ids ? a->out_sorted_token_ids : b.sorted_token_ids;
   int32_t* inv = a->out_inv_perm ? a->out_inv_perm : b.inv_perm;
   const int R = a->M * a->k;
+  hipStream_t main_s = (hipStream_t)stream;
+  MOE_REQUIRE(a->routing == MOE_ROUTING_SOFTMAX || a->routing == MOE_ROUTING_SIGMOID_GROUPED, MOE_ERR_BAD_SHAPE,
+              "forward: unknown routing %d", a->routing);
   int rc;
+  if ((rc = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream))) return rc;
+
+  // The shared expert needs only the quantised activations, so it forks here onto a side stream and runs
+  // beside routing, permutation and the routed GEMMs; the combine joins it.  (Event record / wait is also the
+  // pattern a capturing caller's graph turns into a fork and a join.)
+  hipStream_t side = nullptr;
+  hipEvent_t ev = nullptr, ev_join = nullptr;
+  int rc_shared = MOE_OK;
+  if (a->SI) {
+    if ((rc = side_stream(&side))) return rc;
+    if ((rc = moe_check_hip(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "forward: event"))) return rc;
+    if ((rc = moe_check_hip(hipEventCreateWithFlags(&ev_join, hipEventDisableTiming), "forward: event"))) {
+      (void)hipEventDestroy(ev);
+      return rc;
+    }
+    rc = moe_check_hip(hipEventRecord(ev, main_s), "forward: fork");
+    if (!rc) rc = moe_check_hip(hipStreamWaitEvent(side, ev, 0), "forward: fork");
+    (void)hipEventDestroy(ev);   // released once the recorded work has completed
+    if (rc) {
+      (void)hipEventDestroy(ev_join);
+      return rc;
+    }
+    hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
+    rc_shared = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up,
+                                           b.dense_off, 1, a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws_shared,
+                                           b.gemm_ws_shared_bytes, (moe_stream_t)side);
+    if (!rc_shared)
+      rc_shared = moe_gemm_down_fp8(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
+                                    b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
+  }
+  // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
+  auto join = [&](int code) {
+    if (!a->SI) return code;
+    hipError_t e1 = hipEventRecord(ev_join, side);
+    hipError_t e2 = hipStreamWaitEvent(main_s, ev_join, 0);
+    (void)hipEventDestroy(ev_join);
+    if (code) return code;
+    if (rc_shared) return rc_shared;
+    if (e1 != hipSuccess) return moe_check_hip(e1, "forward: join");
+    return moe_check_hip(e2, "forward: join");
+  };
+
   if (a->routing == MOE_ROUTING_SOFTMAX)
     rc = moe_route_softmax_topk(a->logits, a->M, a->E, a->k, a->renorm, idx, w, stream);
-  else if (a->routing == MOE_ROUTING_SIGMOID_GROUPED)
+  else
     rc = moe_route_sigmoid_grouped(a->logits, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
                                    a->routed_scale, idx, w, stream);
-  else
-    return moe_set_error(MOE_ERR_BAD_SHAPE, "forward: unknown routing %d", a->routing);
-  if (rc) return rc;
+  if (rc) return join(rc);
   if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
                         b.permute_ws_bytes, stream)))
-    return rc;
-  if ((rc = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream))) return rc;
+    return join(rc);
   if ((rc = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets,
                                        a->E, R, a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, stream)))
-    return rc;
+    return join(rc);
   if ((rc = moe_gemm_down_fp8(b.hq, b.sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
                               b.gemm_ws, b.gemm_ws_bytes, stream)))
-    return rc;
-  if (a->SI) {
-    hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, b.dense_off, a->M);
-    if ((rc = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up,
-                                         b.dense_off, 1, a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws, b.gemm_ws_bytes,
-                                         stream)))
-      return rc;
-    if ((rc = moe_gemm_down_fp8(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
-                                b.gemm_ws, b.gemm_ws_bytes, stream)))
-      return rc;
-  }
+    return join(rc);
+  if ((rc = join(MOE_OK))) return rc;
   return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, a->M, a->k, a->D, a->out, stream);
 }
