@@ -67,7 +67,7 @@ struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
   float *w, *sx, *sh, *shs;
   uint8_t *xq, *hq, *hsq;
-  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_shared;
+  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared;
   size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, total;
 };
 
@@ -85,7 +85,8 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
   b.permute_ws_bytes = moe_permute_workspace_bytes(M, k, E);
   b.permute_ws = c.take(b.permute_ws_bytes);
   b.gemm_ws_bytes = moe_gemm_workspace_bytes((int)R, E, I > D ? I : D);
-  b.gemm_ws = c.take(b.gemm_ws_bytes);
+  b.gemm_ws = c.take(b.gemm_ws_bytes);        // work list of the routed gate/up GEMM
+  b.gemm_ws_down = c.take(b.gemm_ws_bytes);   // ... of the routed down GEMM (both are listed in one launch)
   // the shared expert runs beside the routed ones on its own stream: its launches need their own work lists
   b.gemm_ws_shared_bytes = SI ? moe_gemm_workspace_bytes(M, 1, SI > D ? SI : D) : 0;
   b.gemm_ws_shared = SI ? c.take(b.gemm_ws_shared_bytes) : nullptr;
@@ -186,11 +187,14 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
                         b.permute_ws_bytes, stream)))
     return join(rc);
-  if ((rc = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets,
-                                       a->E, R, a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, stream)))
+  if ((rc = moe_gemm_build_lists(b.group_offsets, a->E, R, a->D, a->I, b.gemm_ws, b.gemm_ws_down, b.gemm_ws_bytes,
+                                 stream)))
     return join(rc);
-  if ((rc = moe_gemm_down_fp8(b.hq, b.sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
-                              b.gemm_ws, b.gemm_ws_bytes, stream)))
+  if ((rc = moe_gemm_gateup_impl(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets, a->E, R,
+                                 a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
+    return join(rc);
+  if ((rc = moe_gemm_down_impl(b.hq, b.sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
+                               b.gemm_ws_down, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;
   return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, a->M, a->k, a->D, a->out, stream);

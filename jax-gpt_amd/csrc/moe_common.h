@@ -18,6 +18,17 @@ typedef unsigned short bf16_t;  // raw bf16 bits
 int moe_set_error(int code, const char* fmt, ...);
 int moe_check_hip(hipError_t e, const char* what);
 
+// grouped GEMMs with an optional pre-built work list (moe_gemm.hip); the extern "C" entry points build their own
+int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
+                         size_t ws_bytes_each, moe_stream_t stream);
+int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
+                         const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
+                         int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,
+                         moe_stream_t stream);
+int moe_gemm_down_impl(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
+                       const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
+                       size_t ws_bytes, bool list_built, moe_stream_t stream);
+
 #define MOE_REQUIRE(cond, code, ...) \
   do {                               \
     if (!(cond)) return moe_set_error(code, __VA_ARGS__); \

@@ -70,9 +70,19 @@ __device__ __forceinline__ int tile_rows(int rows, int bm) {
   const int t = (rows + bm - 1) / bm;
   return t <= 1 ? bm : (((rows + t - 1) / t + 15) & ~15);
 }
-__global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __restrict__ group_offsets, int E,
-                                                          int n_col_blocks, int bm, int max_items,
-                                                          WorkHeader* __restrict__ hdr, WorkItem* __restrict__ items) {
+struct ListSpec {
+  int n_col_blocks, max_items;
+  WorkHeader* hdr;
+  WorkItem* items;
+};
+// workgroup b builds list b (the gate/up and the down GEMM of one layer walk the same rows with different
+// column-block counts: one launch lists both)
+__global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __restrict__ group_offsets, int E, int bm,
+                                                          ListSpec l0, ListSpec l1) {
+  const ListSpec spec = blockIdx.x == 0 ? l0 : l1;
+  const int n_col_blocks = spec.n_col_blocks, max_items = spec.max_items;
+  WorkHeader* __restrict__ hdr = spec.hdr;
+  WorkItem* __restrict__ items = spec.items;
   __shared__ int tile_prefix[1025];
   __shared__ int wave_tot[16];
   const int e = threadIdx.x;
@@ -497,6 +507,8 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
   }
 }
 
+int col_blocks(int mode, int N) { return mode == MODE_GATEUP ? N / 128 : (N + 255) / 256; }
+
 int max_items_for(int R, int E, int n_col_blocks, int bm) {
   long long tiles = (long long)(R + bm - 1) / bm + (E < R ? E : R);
   return (int)(tiles * n_col_blocks);
@@ -505,13 +517,16 @@ int max_items_for(int R, int E, int n_col_blocks, int bm) {
 template <int MODE, int XW>
 int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
                const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
-               void* out, float* out_scale, void* ws, hipStream_t s) {
+               void* out, float* out_scale, void* ws, bool list_built, hipStream_t s) {
   using C = Cfg<XW>;
-  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
+  const int ncb = col_blocks(MODE, N);
   const int max_items = max_items_for(R, E, ncb, C::BM);
   WorkHeader* hdr = (WorkHeader*)ws;
   WorkItem* items = (WorkItem*)((char*)ws + sizeof(WorkHeader));
-  hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, ncb, C::BM, max_items, hdr, items);
+  if (!list_built) {
+    const ListSpec spec{ncb, max_items, hdr, items};
+    hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, C::BM, spec, spec);
+  }
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t err = hipFuncSetAttribute((const void*)grouped_gemm_kernel<MODE, XW>,
@@ -534,21 +549,24 @@ int forced_xw() {
   return v == 128 ? 1 : v == 256 ? 2 : 0;
 }
 
+// 256-row tiles once the average expert has more than 128 rows, 128-row tiles otherwise
+int tile_config(int R, int E) { return forced_xw() ? forced_xw() : ((long long)R > 128ll * E ? 2 : 1); }
+
 template <int MODE>
 int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
            const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
-           void* out, float* out_scale, void* ws, size_t ws_bytes, hipStream_t s) {
+           void* out, float* out_scale, void* ws, size_t ws_bytes, bool list_built, hipStream_t s) {
   const size_t need = moe_gemm_workspace_bytes(R, E, N);
   MOE_REQUIRE(ws_bytes >= need, MOE_ERR_WORKSPACE_TOO_SMALL, "gemm: workspace %zu < %zu", ws_bytes, need);
   MOE_REQUIRE(K <= MAX_KB * BK, MOE_ERR_BAD_SHAPE, "gemm: contraction length %d exceeds %d", K, MAX_KB * BK);
   MOE_REQUIRE((long long)N * K <= (1ll << 32) && (long long)R * K <= (1ll << 32), MOE_ERR_BAD_SHAPE,
               "gemm: one expert matrix and the activation array must each stay within 4 GB (N=%d K=%d R=%d)", N, K, R);
   if (R == 0) return MOE_OK;
-  // 256-row tiles once the average expert has more than 128 rows, 128-row tiles otherwise
-  const int xw = forced_xw() ? forced_xw() : ((long long)R > 128ll * E ? 2 : 1);
-  if (xw == 2)
-    return launch_cfg<MODE, 2>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws, s);
-  return launch_cfg<MODE, 1>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws, s);
+  if (tile_config(R, E) == 2)
+    return launch_cfg<MODE, 2>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
+                               list_built, s);
+  return launch_cfg<MODE, 1>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
+                             list_built, s);
 }
 
 }  // namespace
@@ -559,11 +577,10 @@ extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
   return sizeof(WorkHeader) + (size_t)max_items_for(R, E, ncb, 128) * sizeof(WorkItem) + 256;
 }
 
-extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
-                                          const uint8_t* w_gate, const float* sw_gate, const uint8_t* w_up,
-                                          const float* sw_up, const int32_t* group_offsets, int E, int R, int D,
-                                          int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes,
-                                          moe_stream_t stream) {
+int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
+                         const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
+                         int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,
+                         moe_stream_t stream) {
   MOE_REQUIRE(xq && sx && w_gate && sw_gate && w_up && sw_up && group_offsets && hq && sh && ws, MOE_ERR_NULL,
               "gemm_gateup: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0 && D > 0 && I > 0 && D % 128 == 0 && I % 128 == 0, MOE_ERR_BAD_SHAPE,
@@ -571,17 +588,49 @@ extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, co
   MOE_REQUIRE(MOE_ALIGNED16(xq) && MOE_ALIGNED16(w_gate) && MOE_ALIGNED16(w_up) && MOE_ALIGNED16(hq) && MOE_ALIGNED16(ws),
               MOE_ERR_BAD_ALIGN, "gemm_gateup: pointers must be 16-byte aligned");
   return launch<MODE_GATEUP>(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
-                             ws_bytes, (hipStream_t)stream);
+                             ws_bytes, list_built, (hipStream_t)stream);
 }
 
-extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
-                                 const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
-                                 size_t ws_bytes, moe_stream_t stream) {
+extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+                                          const uint8_t* w_gate, const float* sw_gate, const uint8_t* w_up,
+                                          const float* sw_up, const int32_t* group_offsets, int E, int R, int D,
+                                          int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes,
+                                          moe_stream_t stream) {
+  return moe_gemm_gateup_impl(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
+                              ws_bytes, false, stream);
+}
+
+int moe_gemm_down_impl(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
+                       const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
+                       size_t ws_bytes, bool list_built, moe_stream_t stream) {
   MOE_REQUIRE(hq && sh && w_down && sw_down && group_offsets && y_bf16 && ws, MOE_ERR_NULL, "gemm_down: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0 && D > 0 && I > 0 && D % 128 == 0 && I % 128 == 0, MOE_ERR_BAD_SHAPE,
               "gemm_down: need D %% 128 == 0 and I %% 128 == 0 and 1 <= E <= 1024, got E=%d R=%d I=%d D=%d", E, R, I, D);
   MOE_REQUIRE(MOE_ALIGNED16(hq) && MOE_ALIGNED16(w_down) && MOE_ALIGNED16(y_bf16) && MOE_ALIGNED16(ws), MOE_ERR_BAD_ALIGN,
               "gemm_down: pointers must be 16-byte aligned");
   return launch<MODE_DOWN>(hq, sh, nullptr, w_down, sw_down, nullptr, nullptr, group_offsets, E, R, I, D, y_bf16,
-                           nullptr, ws, ws_bytes, (hipStream_t)stream);
+                           nullptr, ws, ws_bytes, list_built, (hipStream_t)stream);
+}
+
+extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
+                                 const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
+                                 size_t ws_bytes, moe_stream_t stream) {
+  return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, stream);
+}
+
+// Lists the work items of a layer's gate/up GEMM (into ws_gateup) and down GEMM (into ws_down) in one launch;
+// the *_impl entry points then take list_built = true.
+int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
+                         size_t ws_bytes_each, moe_stream_t stream) {
+  MOE_REQUIRE(ws_bytes_each >= moe_gemm_workspace_bytes(R, E, I > D ? I : D), MOE_ERR_WORKSPACE_TOO_SMALL,
+              "gemm lists: workspace too small");
+  if (R == 0) return MOE_OK;
+  const int bm = tile_config(R, E) == 2 ? 256 : 128;
+  const int ncb_a = col_blocks(MODE_GATEUP, I), ncb_b = col_blocks(MODE_DOWN, D);
+  const ListSpec a{ncb_a, max_items_for(R, E, ncb_a, bm), (WorkHeader*)ws_gateup,
+                   (WorkItem*)((char*)ws_gateup + sizeof(WorkHeader))};
+  const ListSpec b{ncb_b, max_items_for(R, E, ncb_b, bm), (WorkHeader*)ws_down,
+                   (WorkItem*)((char*)ws_down + sizeof(WorkHeader))};
+  hipLaunchKernelGGL(build_items_kernel, dim3(2), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, bm, a, b);
+  return moe_check_hip(hipGetLastError(), "gemm lists launch");
 }

@@ -2,7 +2,7 @@
 //
 // Replaces jax_gpt/models/qwen35/moe.py:58-80 (_sort_and_group: argsort of the
 // flat expert ids, the scatter-add histogram, and the gathers of token ids).
-// Three launches, all integer work:
+// Three launches (one fused launch when the whole list fits one chunk), all integer work:
 //   1. per-chunk histograms: each wavefront counts its 64 entries with ballot
 //      match masks and adds them to an LDS histogram of the chunk;
 //   2. one workgroup turns the (chunks x E) counts into group sizes, group
@@ -130,6 +130,83 @@ __global__ __launch_bounds__(kThreads) void scatter_kernel(const int32_t* __rest
   }
 }
 
+// R <= kChunk: the three steps in one workgroup, one launch (decode-sized batches are launch-bound).
+__global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* __restrict__ ids, int R, int E, int k,
+                                                                int32_t* __restrict__ group_sizes,
+                                                                int32_t* __restrict__ group_offsets,
+                                                                int32_t* __restrict__ sorted_token_ids,
+                                                                int32_t* __restrict__ sort_order,
+                                                                int32_t* __restrict__ inv_perm) {
+  __shared__ int hist[kMaxE];   // counts, then next free output position per expert
+  __shared__ int wave_tot[kWaves];
+  for (int e = threadIdx.x; e < kMaxE; e += kThreads) hist[e] = 0;
+  __syncthreads();
+  const int bits = ilog2_ceil(E);
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  int my_id[kRounds];
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int f = r * kThreads + threadIdx.x;
+    int id = f < R ? ids[f] : -1;
+    if (id >= E) id = -1;
+    my_id[r] = id;
+    const unsigned long long m = match_any(id, bits);
+    if (id >= 0 && (m & ((1ull << lane) - 1ull)) == 0ull) atomicAdd(&hist[id], __popcll(m));
+  }
+  __syncthreads();
+  // exclusive scan over experts: thread t owns experts [4t, 4t + 4)
+  constexpr int kPer = kMaxE / kThreads;
+  int c[kPer], sum = 0;
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    c[i] = hist[threadIdx.x * kPer + i];
+    sum += c[i];
+  }
+  int incl = sum;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(incl, off, MOE_WAVE);
+    if (lane >= off) incl += o;
+  }
+  if (lane == 63) wave_tot[wv] = incl;
+  __syncthreads();
+  int run = incl - sum;
+  for (int i = 0; i < wv; ++i) run += wave_tot[i];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int e = threadIdx.x * kPer + i;
+    if (e < E) {
+      group_sizes[e] = c[i];
+      group_offsets[e] = run;
+      if (e == E - 1) group_offsets[E] = run + c[i];
+    }
+    hist[e] = run;
+    run += c[i];
+  }
+  __syncthreads();
+  if (!sorted_token_ids && !sort_order && !inv_perm) return;
+#pragma unroll
+  for (int r = 0; r < kRounds; ++r) {
+    const int f = r * kThreads + threadIdx.x;
+    const int id = my_id[r];
+    const unsigned long long m = match_any(id, bits);
+    const int rank = __popcll(m & ((1ull << lane) - 1ull));
+    const int cnt = __popcll(m);
+    int pos = 0;
+    for (int turn = 0; turn < kWaves; ++turn) {   // waves take their turn in flat-index order so ranks stay stable
+      if (wv == turn && id >= 0) pos = hist[id] + rank;
+      __syncthreads();
+      if (wv == turn && id >= 0 && rank == 0) hist[id] += cnt;
+      __syncthreads();
+    }
+    if (id >= 0) {
+      if (sort_order) sort_order[pos] = f;
+      if (sorted_token_ids) sorted_token_ids[pos] = f / k;
+      if (inv_perm) inv_perm[f] = pos;
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" size_t moe_permute_workspace_bytes(int M, int k, int E) {
@@ -152,6 +229,11 @@ extern "C" int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* gro
   const int R = M * k;
   int n_chunks = (R + kChunk - 1) / kChunk;
   if (n_chunks < 1) n_chunks = 1;
+  if (R <= kChunk) {
+    hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(kThreads), 0, s, idx, R, E, k, group_sizes, group_offsets,
+                       sorted_token_ids, sort_order, inv_perm);
+    return moe_check_hip(hipGetLastError(), "permute launch");
+  }
   int32_t* chunk_hist = (int32_t*)ws;
   hipLaunchKernelGGL(hist_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, chunk_hist);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kMaxE), 0, s, chunk_hist, n_chunks, E, group_sizes, group_offsets);
