@@ -117,6 +117,34 @@ def run_workload(jg, torch, name, cfg, layer, steps, warmup):
     res = dict(workload=name, ms_per_step=ev_ms, wall_ms_per_step=wall_ms, flops=flops, tflops=flops / ev_ms / 1e9,
                touched_experts=touched, weight_bytes=weight_bytes, gbs=weight_bytes / ev_ms / 1e6)
 
+    # the same step captured once in a HIP graph and replayed (no per-launch host work): matters for
+    # decode-sized batches, where a dozen dependent launches share a millisecond
+    res["graph_ms_per_step"] = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                jg.moe_experts(x, logits, **kw)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out_g = jg.moe_experts(x, logits, **kw)
+        graph.replay()
+        torch.cuda.synchronize()
+        if not torch.equal(out_g, out):
+            raise RuntimeError("graph replay differs from the eager result")
+        g_ms, _ = timed(torch, graph.replay, steps, 2)
+        if not torch.equal(out_g, out):
+            raise RuntimeError("graph replay differs from the eager result after the timed replays")
+        res["graph_ms_per_step"] = g_ms
+        res["graph_gbs"] = weight_bytes / g_ms / 1e6
+        res["graph_tflops"] = flops / g_ms / 1e9
+        del graph, out_g
+    except Exception as exc:  # noqa: BLE001 - the eager figure stands on its own
+        log(f"graph replay measurement skipped: {exc!r}")
+
     # the dominant kernel alone: the routed launch of the gate/up grouped GEMM, HIP events on the
     # stream it is launched on (torch's current stream is the stream handed to the C ABI)
     sg = jg.permute(dbg["indices"], E)
@@ -209,12 +237,14 @@ def main():
         "config": {"workload": args.workload, **{k: cfg[k] for k in ("M", "D", "E", "k", "I", "SI", "routing")},
                    "touched_experts": main_res["touched_experts"]},
         "frac_of_peak": (value / PEAK_HBM_GBS) if is_decode else (value / PEAK_FP8_TFLOPS),
+        "graph_replay_ms_per_step": main_res["graph_ms_per_step"],
         "roofline": roof,
     }
     if decode:
         dk = decode["gateup_kernel"]
         line["decode"] = {"metric": "HBM GB/s over touched fp8 expert weights", "value": decode["gbs"], "unit": "GB/s",
-                          "ms_per_step": decode["ms_per_step"], "touched_experts": decode["touched_experts"],
+                          "ms_per_step": decode["ms_per_step"], "graph_replay_ms_per_step": decode["graph_ms_per_step"],
+                          "graph_replay_value": decode.get("graph_gbs"), "touched_experts": decode["touched_experts"],
                           "weight_bytes": decode["weight_bytes"], "frac_of_peak": decode["gbs"] / PEAK_HBM_GBS,
                           "roofline": {"bound": "hbm", "achieved": dk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                        "frac": dk["gbs"] / PEAK_HBM_GBS, "traffic": None,

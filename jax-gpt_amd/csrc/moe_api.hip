@@ -136,35 +136,41 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   MOE_REQUIRE(a->routing == MOE_ROUTING_SOFTMAX || a->routing == MOE_ROUTING_SIGMOID_GROUPED, MOE_ERR_BAD_SHAPE,
               "forward: unknown routing %d", a->routing);
   int rc;
-  if ((rc = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream))) return rc;
 
-  // The shared expert needs only the quantised activations, so it forks here onto a side stream and runs
-  // beside routing, permutation and the routed GEMMs; the combine joins it.  (Event record / wait is also the
-  // pattern a capturing caller's graph turns into a fork and a join.)
+  // With a shared expert the call forks at once: the side stream quantises the activations and runs the shared
+  // expert, while the caller's stream routes, permutes and lists the work; the routed gate/up GEMM waits for
+  // the quantised activations, the combine for the shared expert's output.  (Event record / wait is also the
+  // pattern a capturing caller's graph turns into forks and joins.)
   hipStream_t side = nullptr;
-  hipEvent_t ev = nullptr, ev_join = nullptr;
+  hipEvent_t ev_fork = nullptr, ev_quant = nullptr, ev_join = nullptr;
   int rc_shared = MOE_OK;
+  bool quant_joined = true;
   if (a->SI) {
     if ((rc = side_stream(&side))) return rc;
-    if ((rc = moe_check_hip(hipEventCreateWithFlags(&ev, hipEventDisableTiming), "forward: event"))) return rc;
-    if ((rc = moe_check_hip(hipEventCreateWithFlags(&ev_join, hipEventDisableTiming), "forward: event"))) {
-      (void)hipEventDestroy(ev);
-      return rc;
+    hipError_t e = hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ev_quant, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ev_join, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventRecord(ev_fork, main_s);
+    if (e == hipSuccess) e = hipStreamWaitEvent(side, ev_fork, 0);
+    if (ev_fork) (void)hipEventDestroy(ev_fork);   // released once the recorded work has completed
+    if (e != hipSuccess) {
+      if (ev_quant) (void)hipEventDestroy(ev_quant);
+      if (ev_join) (void)hipEventDestroy(ev_join);
+      return moe_check_hip(e, "forward: fork");
     }
-    rc = moe_check_hip(hipEventRecord(ev, main_s), "forward: fork");
-    if (!rc) rc = moe_check_hip(hipStreamWaitEvent(side, ev, 0), "forward: fork");
-    (void)hipEventDestroy(ev);   // released once the recorded work has completed
-    if (rc) {
-      (void)hipEventDestroy(ev_join);
-      return rc;
-    }
+    quant_joined = false;
+    rc_shared = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, (moe_stream_t)side);
+    if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
-    rc_shared = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up,
-                                           b.dense_off, 1, a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws_shared,
-                                           b.gemm_ws_shared_bytes, (moe_stream_t)side);
+    if (!rc_shared)
+      rc_shared = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up,
+                                             b.dense_off, 1, a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws_shared,
+                                             b.gemm_ws_shared_bytes, (moe_stream_t)side);
     if (!rc_shared)
       rc_shared = moe_gemm_down_fp8(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
                                     b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
+  } else {
+    if ((rc = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream))) return rc;
   }
   // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
   auto join = [&](int code) {
@@ -172,6 +178,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     hipError_t e1 = hipEventRecord(ev_join, side);
     hipError_t e2 = hipStreamWaitEvent(main_s, ev_join, 0);
     (void)hipEventDestroy(ev_join);
+    (void)hipEventDestroy(ev_quant);
     if (code) return code;
     if (rc_shared) return rc_shared;
     if (e1 != hipSuccess) return moe_check_hip(e1, "forward: join");
@@ -190,6 +197,10 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   if ((rc = moe_gemm_build_lists(b.group_offsets, a->E, R, a->D, a->I, b.gemm_ws, b.gemm_ws_down, b.gemm_ws_bytes,
                                  stream)))
     return join(rc);
+  if (!quant_joined) {
+    if (rc_shared) return join(rc_shared);
+    if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
+  }
   if ((rc = moe_gemm_gateup_impl(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets, a->E, R,
                                  a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);

@@ -143,9 +143,12 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
   __syncthreads();
   const int bits = ilog2_ceil(E);
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const int rounds = (R + kThreads - 1) / kThreads;   // uniform; the rounds past the end have nothing to place
   int my_id[kRounds];
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) {
+    my_id[r] = -1;
+    if (r >= rounds) continue;
     const int f = r * kThreads + threadIdx.x;
     int id = f < R ? ids[f] : -1;
     if (id >= E) id = -1;
@@ -187,6 +190,7 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
   if (!sorted_token_ids && !sort_order && !inv_perm) return;
 #pragma unroll
   for (int r = 0; r < kRounds; ++r) {
+    if (r >= rounds) break;
     const int f = r * kThreads + threadIdx.x;
     const int id = my_id[r];
     const unsigned long long m = match_any(id, bits);

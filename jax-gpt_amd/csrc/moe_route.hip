@@ -136,6 +136,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
   const int per = E / n_group;
   float score[VPL];
   unsigned long long key[VPL];
+  int gid[VPL];   // group of each slot's expert (one integer division per slot, not one per group and slot)
 #pragma unroll
   for (int s = 0; s < VPL; ++s) {
     int e = lane + 64 * s;
@@ -143,6 +144,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
     score[s] = ok ? sigmoid_det(row[e]) : 0.f;
     float choice = __fadd_rn(score[s], (ok && bias) ? bias[e] : 0.f);
     key[s] = ok ? make_key(choice, (unsigned)e) : 0ull;
+    gid[s] = ok ? e / per : -1;
   }
   // group score = sum of the two best choice scores of the group (lane g keeps group g's)
   unsigned long long gkey = 0ull;
@@ -150,7 +152,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
     unsigned long long b1 = 0ull, b2 = 0ull;
 #pragma unroll
     for (int s = 0; s < VPL; ++s) {
-      bool in = (lane + 64 * s) / per == g;
+      bool in = gid[s] == g;
       b1 = (in && key[s] > b1) ? key[s] : b1;
     }
     b1 = wave_max_u64(b1);
@@ -158,7 +160,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
     if (per >= 2) {
 #pragma unroll
       for (int s = 0; s < VPL; ++s) {
-        bool in = (lane + 64 * s) / per == g && key[s] < b1;
+        bool in = gid[s] == g && key[s] < b1;
         b2 = (in && key[s] > b2) ? key[s] : b2;
       }
       b2 = wave_max_u64(b2);
@@ -174,8 +176,8 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
   }
 #pragma unroll
   for (int s = 0; s < VPL; ++s) {
-    int g = (lane + 64 * s) / per;
-    if (g >= n_group || !((keep >> g) & 1ull)) key[s] = 0ull;
+    const int g = gid[s];
+    if (g < 0 || g >= n_group || !((keep >> g) & 1ull)) key[s] = 0ull;
   }
   int my_idx = 0;
   float my_w = 0.f, wsum = 0.f;

@@ -273,3 +273,41 @@ def test_reference_entry_points(jg):
     ref_routed = O.combine(ref["y"], ref["weights"], ref["inv_perm"])
     H.assert_close_out(H.bf16_to_np(routed), ref_routed, inner=256)
     H.assert_close_out(H.bf16_to_np(shared), ref["shared_out"], inner=128)
+
+
+def test_graph_replay_matches_eager(jg):
+    """The whole path (side stream for the shared expert included) captured in a HIP graph: every replay, with
+    eager calls and synchronisations between the replays, gives the eager result bit for bit."""
+    import torch
+    _say("graph replay")
+    prob = H.make_problem(M=64, D=512, E=32, k=4, I=256, SI=256, seed=7, routing="sigmoid_grouped")
+    ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
+    x = H.to_bf16_cuda(prob["x"]); lg = H.to_cuda(prob["logits"])
+    kw = dict(top_k=4, experts=ex, shared=sh, routing="sigmoid_grouped", n_group=4, topk_group=2)
+    eager = jg.moe_experts(x, lg, **kw)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        jg.moe_experts(x, lg, **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = jg.moe_experts(x, lg, **kw)
+    for i in range(4):
+        _say("   replay", i)
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {i} differs"
+        again = jg.moe_experts(x, lg, **kw)           # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(again, eager)
+    # new inputs in the captured buffers are picked up by the next replay
+    x2 = H.to_bf16_cuda(prob["x"][::-1].copy())
+    want = jg.moe_experts(x2, lg, **kw)
+    x.copy_(x2)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
