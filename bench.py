@@ -27,7 +27,7 @@ PEAK_FP8_TFLOPS = 5000.0     # MI355X dense fp8 MFMA (published)
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E (published)
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (counter x calibration factor; the summary and the commands are in profiles/).  None = not measured.
-MEASURED_TRAFFIC = {"deepseek_v3_prefill": 12163e6 + 160e6}
+MEASURED_TRAFFIC = {"deepseek_v3_prefill": 8536e6 + 143e6}
 
 WORKLOADS = {
     # BASELINE config 3 / 4: DeepSeek-V3-style layer
@@ -227,7 +227,7 @@ def main():
         metric, value, unit = "MoE layer fp8 TFLOP/s (prefill)", main_res["tflops"], "TFLOP/s"
         roof = {"bound": "mfma", "achieved": gk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                 "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC.get(args.workload),
-                "kernel": "grouped_gemm_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
+                "kernel": "grouped_gemm_kernel<0, 2>, routed launch (gate/up + SwiGLU + h quantisation)",
                 "algorithmic_bytes_per_launch": gk["bytes_per_launch"],
                 "avg_launch_ms": gk["avg_launch_ms"], "flops_per_launch": gk["flops_per_launch"]}
     line = {

@@ -163,6 +163,9 @@ struct Cfg {
   static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // 151040 / 133120
   static constexpr int X_DMA = 2 * XW;                         // 1 KB activation row groups per wave per step
   static constexpr int VM_PER_STEP = 4 + X_DMA + 1;            // + 4 weight row groups + 1 scale copy
+  // skip the copies of activation rows past the end of a short tile; only where every step waits for all of its
+  // copies anyway (PRE == 1), so that no wait has to count a varying number of them
+  static constexpr bool XSKIP = PRE == 1;
   // MFMA groups by which wave set 1 trails wave set 0 (build-time tuning knobs; measured best: half a step at
   // BM = 128, one group at BM = 256 where registers are short)
 #ifndef MOE_ROT1
@@ -275,11 +278,18 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     if (row_ids) g = row_ids[g];
     soff = (unsigned)g * (unsigned)KB * 4u;
   }
+  // With XSKIP, activation row groups that lie wholly past the item's last row are not copied (their LDS rows
+  // keep stale bytes; whatever the matrix cores make of them lands in rows the epilogue never stores).  The valid
+  // groups of a wave are a prefix of its X_DMA groups.
+  const int nxv = C::XSKIP ? min(C::X_DMA, max(0, ((item.row_count + 7) >> 3) - wave * C::X_DMA)) : C::X_DMA;
   // copy operation i (0 <= i < VM_PER_STEP) of K step kb
   auto issue_op = [&](int kb, int i) {
     uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
     if (i < 4) dma16(wmat + (size_t)kb * BK, woff[i], st + (wave * 4 + i) * 1024);
-    else if (i < 4 + C::X_DMA) dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + (wave * C::X_DMA + i - 4) * 1024);
+    else if (i < 4 + C::X_DMA) {
+      if (!C::XSKIP || i - 4 < nxv)
+        dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + (wave * C::X_DMA + i - 4) * 1024);
+    }
     else if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4);
   };
   auto issue = [&](int kb) {
