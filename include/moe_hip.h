@@ -93,13 +93,25 @@ int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
                       int D, void* y_bf16, void* ws, size_t ws_bytes, moe_stream_t stream);
 
 /* moe.py:90-94 (_scatter_back) as a deterministic gather: out[t] = sum_s w[t,s] *
- * y[inv_perm[t*k+s]] (+ shared[t]) in f32, one bf16 rounding.  shared may be NULL
- * (moe.py:281 adds the shared expert's output). */
+ * y[inv_perm[t*k+s]] (+ shared_gate[t] * shared[t]) in f32, one bf16 rounding.  shared may be
+ * NULL (moe.py:281 adds the shared expert's output); shared_gate may be NULL (= 1; moe.py:278-279
+ * multiplies the shared expert's output by sigmoid(x @ shared_expert_gate_weight)). */
 int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
-                const void* shared_bf16, int M, int k, int D, void* out_bf16, moe_stream_t stream);
+                const void* shared_bf16, const float* shared_gate, int M, int k, int D, void* out_bf16,
+                moe_stream_t stream);
+
+/* moe.py:50 (logits = matmul_maybe_fp8(x, gate_weight), a bf16 matmul widened to f32 by :51) and
+ * moe.py:278 (sigmoid(x @ shared_expert_gate_weight)).  w_router is (E, D) bf16, K-contiguous (the
+ * checkpoint layout of mlp.gate.weight; the reference's in-memory array is its transpose (D, E));
+ * w_shared_gate is (1, D) bf16 or NULL.  logits (M, E) f32 hold bf16-rounded values; shared_gate
+ * (M) f32 holds bf16-rounded sigmoids (NULL iff w_shared_gate is NULL). */
+size_t moe_router_workspace_bytes(int M, int D, int E);
+int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
+                      const void* w_shared_gate_bf16, float* logits, float* shared_gate, void* ws,
+                      size_t ws_bytes, moe_stream_t stream);
 
 /* The whole path (moe.py:97-114 + 225-232 + 281): router logits in, combined hidden
- * states out. */
+ * states out -- or, with w_router set, hidden states in (moe.py:235-282, moe_layer). */
 typedef struct MoeForwardArgs {
   int M, D, E, k, I;       /* tokens, hidden, routed experts, top-k, expert intermediate */
   int SI;                  /* shared-expert intermediate, 0 = no shared expert */
@@ -108,7 +120,7 @@ typedef struct MoeForwardArgs {
   int renorm;
   float routed_scale;
   const void* x;           /* (M, D) bf16 */
-  const float* logits;     /* (M, E) */
+  const float* logits;     /* (M, E); ignored (may be NULL) when w_router is set */
   const float* bias;       /* (E) or NULL */
   const uint8_t *w_gate, *w_up, *w_down;    /* (E,I,D) (E,I,D) (E,D,I) */
   const float *sw_gate, *sw_up, *sw_down;
@@ -121,6 +133,11 @@ typedef struct MoeForwardArgs {
   int32_t* out_group_sizes;      /* (E) */
   int32_t* out_sorted_token_ids; /* (R) */
   int32_t* out_inv_perm;         /* (R) */
+  /* router in front of the path (NULL = the caller supplies logits) */
+  const void* w_router;          /* (E, D) bf16: logits = bf16(x . w_router^T), moe.py:50 */
+  const void* w_shared_gate;     /* (1, D) bf16 or NULL: shared expert's output is scaled by
+                                    sigmoid(x . w_shared_gate^T), moe.py:278-279; needs w_router and SI > 0 */
+  float* out_logits;             /* (M, E) optional debug output of the computed logits */
 } MoeForwardArgs;
 
 size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI);

@@ -19,6 +19,7 @@ from .moe import (  # noqa: F401
     quant_act,
     quantize_weight_block,
     route_sigmoid_grouped,
+    router_logits,
     route_softmax_topk,
     shared_expert_forward,
 )

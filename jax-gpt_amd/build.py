@@ -15,7 +15,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libmoe_hip.so")
 
-SOURCES = ["moe_api.hip", "moe_route.hip", "moe_permute.hip", "moe_quant.hip", "moe_gemm.hip",
+SOURCES = ["moe_api.hip", "moe_route.hip", "moe_router.hip", "moe_permute.hip", "moe_quant.hip", "moe_gemm.hip",
            "moe_combine.hip"]
 # no v_pk_*_f32 code generation (some packed-f32 forms misbehave on this hardware pool)
 COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
@@ -23,6 +23,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-
           "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 # routing and combine promise individually rounded f32 operations (bit-reproducible on a CPU)
 PER_FILE = {"moe_route.hip": ["-ffp-contract=off"], "moe_combine.hip": ["-ffp-contract=off"],
+            "moe_router.hip": ["-ffp-contract=off"],
             # MFMA results go straight to VGPRs: the block-scale FMA consumes them on the vector ALU
             "moe_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-Wno-inline-asm"]}   # m0 is clobbered on purpose
 

@@ -24,7 +24,7 @@ int moe_check_hip(hipError_t e, const char* what) {
   return moe_set_error(MOE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-extern "C" int moe_abi_version(void) { return 1; }
+extern "C" int moe_abi_version(void) { return 2; }
 extern "C" const char* moe_last_error(void) { return g_err; }
 
 namespace {
@@ -65,13 +65,13 @@ struct Carver {
 
 struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
-  float *w, *sx, *sh, *shs;
+  float *w, *sx, *sh, *shs, *logits, *shared_gate;
   uint8_t *xq, *hq, *hsq;
-  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared;
-  size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, total;
+  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared, *router_ws;
+  size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, router_ws_bytes, total;
 };
 
-ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
+ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool router) {
   ForwardBuffers b;
   Carver c{(char*)ws, 0};
   const size_t R = (size_t)M * k;
@@ -98,6 +98,10 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
   b.hsq = SI ? (uint8_t*)c.take((size_t)M * SI) : nullptr;
   b.shs = SI ? (float*)c.take((size_t)M * (SI / 128) * 4) : nullptr;
   b.ys = SI ? c.take((size_t)M * D * 2) : nullptr;
+  b.logits = router ? (float*)c.take((size_t)M * E * 4) : nullptr;
+  b.shared_gate = router ? (float*)c.take((size_t)M * 4) : nullptr;
+  b.router_ws_bytes = router ? moe_router_workspace_bytes(M, D, E) : 0;
+  b.router_ws = router ? c.take(b.router_ws_bytes) : nullptr;
   b.total = c.used;
   return b;
 }
@@ -106,7 +110,7 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI) {
 
 extern "C" size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI) {
   if (M < 0 || D <= 0 || E <= 0 || k <= 0 || I <= 0 || SI < 0) return 0;
-  return carve(nullptr, M, D, E, k, I, SI).total;
+  return carve(nullptr, M, D, E, k, I, SI, true).total;   // room for the router whether or not a call uses it
 }
 
 extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, moe_stream_t stream) {
@@ -115,7 +119,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
               "forward: bad dims M=%d D=%d E=%d k=%d I=%d SI=%d", a->M, a->D, a->E, a->k, a->I, a->SI);
   MOE_REQUIRE(a->D % 128 == 0 && a->I % 128 == 0 && a->SI % 128 == 0, MOE_ERR_BAD_SHAPE,
               "forward: D=%d, I=%d and SI=%d must be multiples of 128", a->D, a->I, a->SI);
-  MOE_REQUIRE(a->x && a->logits && a->out && a->w_gate && a->w_up && a->w_down && a->sw_gate && a->sw_up && a->sw_down,
+  MOE_REQUIRE(a->x && (a->logits || a->w_router) && a->out && a->w_gate && a->w_up && a->w_down && a->sw_gate && a->sw_up && a->sw_down,
               MOE_ERR_NULL, "forward: null tensor pointer");
   if (a->SI)
     MOE_REQUIRE(a->ws_gate && a->ws_up && a->ws_down && a->sws_gate && a->sws_up && a->sws_down, MOE_ERR_NULL,
@@ -125,7 +129,10 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   MOE_REQUIRE(ws_bytes >= need, MOE_ERR_WORKSPACE_TOO_SMALL, "forward: workspace %zu < %zu", ws_bytes, need);
   if (a->M == 0) return MOE_OK;
 
-  ForwardBuffers b = carve(ws, a->M, a->D, a->E, a->k, a->I, a->SI);
+  MOE_REQUIRE(!a->w_shared_gate || (a->w_router && a->SI), MOE_ERR_NULL,
+              "forward: w_shared_gate needs w_router and a shared expert");
+  MOE_REQUIRE(a->w_router || !a->out_logits, MOE_ERR_NULL, "forward: out_logits is an output of the router (w_router)");
+  ForwardBuffers b = carve(ws, a->M, a->D, a->E, a->k, a->I, a->SI, true);
   int32_t* idx = a->out_idx ? a->out_idx : b.idx;
   float* w = a->out_w ? a->out_w : b.w;
   int32_t* gsz = a->out_group_sizes ? a->out_group_sizes : b.group_sizes;
@@ -185,10 +192,20 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     return moe_check_hip(e2, "forward: join");
   };
 
+  const float* logits = a->logits;
+  const float* shared_gate = nullptr;
+  if (a->w_router) {
+    float* lg = a->out_logits ? a->out_logits : b.logits;
+    if ((rc = moe_router_logits(a->x, a->M, a->D, a->w_router, a->E, a->w_shared_gate, lg,
+                                a->w_shared_gate ? b.shared_gate : nullptr, b.router_ws, b.router_ws_bytes, stream)))
+      return join(rc);
+    logits = lg;
+    if (a->w_shared_gate) shared_gate = b.shared_gate;
+  }
   if (a->routing == MOE_ROUTING_SOFTMAX)
-    rc = moe_route_softmax_topk(a->logits, a->M, a->E, a->k, a->renorm, idx, w, stream);
+    rc = moe_route_softmax_topk(logits, a->M, a->E, a->k, a->renorm, idx, w, stream);
   else
-    rc = moe_route_sigmoid_grouped(a->logits, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
+    rc = moe_route_sigmoid_grouped(logits, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
                                    a->routed_scale, idx, w, stream);
   if (rc) return join(rc);
   if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
@@ -208,5 +225,5 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
                                b.gemm_ws_down, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;
-  return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, a->M, a->k, a->D, a->out, stream);
+  return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, shared_gate, a->M, a->k, a->D, a->out, stream);
 }

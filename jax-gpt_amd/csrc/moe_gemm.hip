@@ -398,7 +398,9 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
       v8i xf[XA + 1];
 #pragma unroll
       for (int j = 0; j < XA; ++j) xf[j] = read_frag(xt + j * 32 * BK);
-      if (ROT > 0 && kb > 0 && (FULL || XF - 1 < jmax)) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
+      if constexpr (ROT > 0) {
+        if (kb > 0 && (FULL || XF - 1 < jmax)) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
+      }
 #pragma unroll
       for (int j = 0; j <= NG; ++j) {
         if (j + XA < NG) xf[(j + XA) % (XA + 1)] = read_frag(xt + (j + XA) * 32 * BK);
@@ -420,7 +422,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
         if (j > 0 && (FULL || j - 1 < jmax)) fm((j - 1) & 1, j - 1, sxv[j - 1] * s0, sxv[j - 1] * s1);
       }
     }
-    if (ROT > 0) {
+    if constexpr (ROT > 0) {
       late(false, 0);
       if (FULL || XF - 1 < jmax) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
     }

@@ -12,29 +12,6 @@
 
 namespace {
 
-__device__ __forceinline__ float exp_det(float x) {
-#pragma clang fp contract(off)
-  x = fminf(fmaxf(x, -87.0f), 88.0f);
-  float n = rintf(__fmul_rn(x, 1.44269504088896341f));
-  float r = __fsub_rn(x, __fmul_rn(n, 0.693145751953125f));
-  r = __fsub_rn(r, __fmul_rn(n, 1.42860682030941723212e-6f));
-  float p = 1.9875691500e-4f;
-  p = __fadd_rn(__fmul_rn(p, r), 1.3981999507e-3f);
-  p = __fadd_rn(__fmul_rn(p, r), 8.3334519073e-3f);
-  p = __fadd_rn(__fmul_rn(p, r), 4.1665795894e-2f);
-  p = __fadd_rn(__fmul_rn(p, r), 1.6666665459e-1f);
-  p = __fadd_rn(__fmul_rn(p, r), 5.0000001201e-1f);
-  float r2 = __fmul_rn(r, r);
-  float y = __fadd_rn(__fmul_rn(p, r2), r);
-  y = __fadd_rn(y, 1.0f);
-  float two_n = __uint_as_float((unsigned)((int)n + 127) << 23);
-  return __fmul_rn(y, two_n);
-}
-
-__device__ __forceinline__ float sigmoid_det(float x) {
-  return __fdiv_rn(1.0f, __fadd_rn(1.0f, exp_det(-x)));
-}
-
 // value-descending, ties -> lower index: larger key wins.  key 0 = absent.
 __device__ __forceinline__ unsigned long long make_key(float v, unsigned idx) {
   unsigned u = __float_as_uint(v + 0.0f);  // -0 -> +0

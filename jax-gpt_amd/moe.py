@@ -225,15 +225,18 @@ def gemm_down(hq, sh, down, group_offsets):
     return y
 
 
-def combine(y, weights, inv_perm, shared=None):
+def combine(y, weights, inv_perm, shared=None, shared_gate=None):
+    """moe.py:90-94 and the add of :281; `shared_gate` (M,) f32 scales the shared rows (moe.py:278-279)."""
     y = _dev(y, torch.bfloat16, "y")
     weights = _dev(weights, torch.float32, "weights")
     inv_perm = _dev(inv_perm, torch.int32, "inv_perm")
     shared = None if shared is None else _dev(shared, torch.bfloat16, "shared")
+    shared_gate = None if shared_gate is None else _dev(shared_gate, torch.float32, "shared_gate")
     M, k = weights.shape
     D = y.shape[1]
     out = _empty((M, D), torch.bfloat16, y)
-    check(lib().moe_combine(_ptr(y), _ptr(weights), _ptr(inv_perm), _ptr(shared), M, k, D, _ptr(out), _stream()))
+    check(lib().moe_combine(_ptr(y), _ptr(weights), _ptr(inv_perm), _ptr(shared), _ptr(shared_gate), M, k, D,
+                            _ptr(out), _stream()))
     return out
 
 
@@ -263,23 +266,81 @@ def shared_expert_forward(x, gate_proj, up_proj, down_proj):
     return gemm_down(hq, sh, down_proj, off)
 
 
+_router_cache = {}
+
+
+def _router_weight(w, name):
+    """The reference keeps router weights input-major, (D, E) / (D, 1) (model.py:83-85, used as x @ w at
+    moe.py:50 and :278); the kernel wants them K-contiguous, (E, D) bf16: transposed once and cached."""
+    if isinstance(w, dict):
+        raise TypeError(f"{name}: an fp8 router weight is not supported; pass the bf16/f32 (D, E) array")
+    if not isinstance(w, torch.Tensor):
+        raise TypeError(f"{name}: expected a tensor")
+    if not w.is_cuda:
+        raise RuntimeError(f"{name}: must live on the GPU (this path has no CPU fallback)")
+    if w.dim() != 2 or w.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"{name}: expected a 2-D bf16/f32 array (D, E), got {tuple(w.shape)} {w.dtype}")
+    key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
+    hit = _router_cache.get(key)
+    if hit is not None and hit[0]() is w:
+        return hit[1]
+    wt = w.t().to(torch.bfloat16).contiguous()
+    _router_cache[key] = (weakref.ref(w), wt)
+    return wt
+
+
+def router_logits(x, gate_weight, shared_expert_gate_weight=None):
+    """moe.py:50 (and :278): logits = bf16(x @ gate_weight) as f32 (M, E); with a shared gate weight (D, 1)
+    also returns sigmoid(bf16(x @ w)) rounded to bf16, as f32 (M,)."""
+    x = _dev(x, torch.bfloat16, "x")
+    wr = _router_weight(gate_weight, "gate_weight")
+    E, D = wr.shape
+    M = x.shape[0]
+    if x.shape[1] != D:
+        raise ValueError(f"gate_weight: expected ({x.shape[1]}, E), got {tuple(gate_weight.shape)}")
+    wsg = None
+    if shared_expert_gate_weight is not None:
+        wsg = _router_weight(shared_expert_gate_weight, "shared_expert_gate_weight")
+        if tuple(wsg.shape) != (1, D):
+            raise ValueError(f"shared_expert_gate_weight: expected ({D}, 1), got {tuple(shared_expert_gate_weight.shape)}")
+    logits = _empty((M, E), torch.float32, x)
+    gate = _empty((M,), torch.float32, x) if wsg is not None else None
+    nbytes = lib().moe_router_workspace_bytes(M, D, E)
+    ws = _empty((max(nbytes, 16),), torch.uint8, x)
+    check(lib().moe_router_logits(_ptr(x), M, D, _ptr(wr), E, _ptr(wsg), _ptr(logits), _ptr(gate), _ptr(ws), nbytes,
+                                  _stream()))
+    return logits if gate is None else (logits, gate)
+
+
 def moe_routing(x, gate_weight, n_experts_per_token):
-    """moe.py:37-55.  The router matmul is not part of this path yet: pass router
-    logits to `moe_experts`, or logits computed by the caller."""
-    raise NotImplementedError(
-        "moe_routing(x, gate_weight, k) needs the router matmul, which this build does not provide yet; "
-        "call route_softmax_topk(router_logits, k) or moe_experts(x, router_logits, ...)")
+    """moe.py:37-55: router matmul, f32 softmax, top-k, renormalise.  x (M, D) bf16, gate_weight (D, E)."""
+    return route_softmax_topk(router_logits(x, gate_weight), n_experts_per_token)
 
 
 def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=None, n_group=1, topk_group=1,
-                renorm=True, routed_scale=1.0, shared=None, return_debug=False):
+                renorm=True, routed_scale=1.0, shared=None, return_debug=False, gate_weight=None,
+                shared_expert_gate_weight=None):
     """Router logits in, combined hidden states out (one C-ABI call, `moe_forward`).
 
     x (M, D) bf16; router_logits (M, E) f32; experts / shared: dicts with keys
     'gate_proj', 'up_proj', 'down_proj' holding block-fp8 dicts (or plain arrays).
+    With `gate_weight` (D, E) the call computes the logits itself (moe.py:50; pass
+    router_logits=None); `shared_expert_gate_weight` (D, 1) then scales the shared
+    expert's output by its sigmoid gate (moe.py:278-279).
     Returns (M, D) bf16, plus a dict of the integer intermediates if return_debug."""
     x = _dev(x, torch.bfloat16, "x")
-    logits = _dev(router_logits, torch.float32, "router_logits")
+    wr = wsg = None
+    if gate_weight is not None:
+        if router_logits is not None:
+            raise ValueError("pass either router_logits or gate_weight, not both")
+        wr = _router_weight(gate_weight, "gate_weight")
+        if shared_expert_gate_weight is not None:
+            wsg = _router_weight(shared_expert_gate_weight, "shared_expert_gate_weight")
+        logits = None
+    else:
+        if shared_expert_gate_weight is not None:
+            raise ValueError("shared_expert_gate_weight needs gate_weight (the router runs inside the call)")
+        logits = _dev(router_logits, torch.float32, "router_logits")
     if routing not in ROUTING:
         raise ValueError(f"routing must be one of {sorted(ROUTING)}, got {routing!r}")
     M, D = x.shape
@@ -287,15 +348,27 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     wu, su = _expert_weight(experts["up_proj"], "up_proj")
     wd, sd = _expert_weight(experts["down_proj"], "down_proj")
     E, I, _ = wg.shape
-    if tuple(logits.shape) != (M, E):
+    if logits is not None and tuple(logits.shape) != (M, E):
         raise ValueError(f"router_logits: expected {(M, E)}, got {tuple(logits.shape)}")
+    if wr is not None and tuple(wr.shape) != (E, D):
+        raise ValueError(f"gate_weight: expected {(D, E)}, got {tuple(gate_weight.shape)}")
+    if wsg is not None and tuple(wsg.shape) != (1, D):
+        raise ValueError(f"shared_expert_gate_weight: expected {(D, 1)}, got {tuple(shared_expert_gate_weight.shape)}")
+    if wsg is not None and shared is None:
+        raise ValueError("shared_expert_gate_weight needs a shared expert")
     if wg.shape != (E, I, D) or wu.shape != (E, I, D) or wd.shape != (E, D, I):
         raise ValueError(f"expert weight shapes {tuple(wg.shape)} {tuple(wu.shape)} {tuple(wd.shape)} do not fit D={D}")
     a = MoeForwardArgs()
     a.M, a.D, a.E, a.k, a.I = M, D, E, top_k, I
     a.routing, a.n_group, a.topk_group, a.renorm, a.routed_scale = ROUTING[routing], n_group, topk_group, int(renorm), routed_scale
-    keep = [x, logits, wg, sg, wu, su, wd, sd]
-    a.x, a.logits = x.data_ptr(), logits.data_ptr()
+    keep = [x, logits, wg, sg, wu, su, wd, sd, wr, wsg]
+    a.x = x.data_ptr()
+    if logits is not None:
+        a.logits = logits.data_ptr()
+    if wr is not None:
+        a.w_router = wr.data_ptr()
+    if wsg is not None:
+        a.w_shared_gate = wsg.data_ptr()
     if bias is not None:
         bias = _dev(bias, torch.float32, "bias")
         keep.append(bias)
@@ -322,6 +395,9 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
         dbg = dict(indices=_empty((M, top_k), torch.int32, x), weights=_empty((M, top_k), torch.float32, x),
                    group_sizes=_empty((E,), torch.int32, x), sorted_token_ids=_empty((R,), torch.int32, x),
                    inv_perm=_empty((R,), torch.int32, x))
+        if wr is not None:
+            dbg["logits"] = _empty((M, E), torch.float32, x)
+            a.out_logits = dbg["logits"].data_ptr()
         a.out_idx, a.out_w = dbg["indices"].data_ptr(), dbg["weights"].data_ptr()
         a.out_group_sizes = dbg["group_sizes"].data_ptr()
         a.out_sorted_token_ids, a.out_inv_perm = dbg["sorted_token_ids"].data_ptr(), dbg["inv_perm"].data_ptr()
@@ -333,6 +409,27 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
 
 
 def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=None):
-    """moe.py:235-282.  Needs the router matmul (see moe_routing)."""
-    raise NotImplementedError("moe_layer needs the router matmul, which this build does not provide yet; "
-                              "use moe_experts(x, router_logits, ...)")
+    """moe.py:235-282: route + routed experts + gated shared expert, (B, T, D) in and out.
+
+    `params` holds the reference's keys (model.py:79-114): gate_weight (D, E); gate_proj, up_proj,
+    down_proj (block-fp8 dicts or plain (E, in, out) arrays); shared_gate_proj, shared_up_proj,
+    shared_down_proj (dicts or plain (in, out) arrays); shared_expert_gate_weight (D, 1).
+    One GPU only: the expert-parallel branch of the reference (moe.py:263-268) is not part of this build."""
+    if n_devices != 1 or mesh is not None:
+        raise NotImplementedError("moe_layer: this build runs on one GPU (n_devices=1, mesh=None)")
+    if x.dim() != 3:
+        raise ValueError(f"x: expected (B, T, D), got {tuple(x.shape)}")
+    B, T, D = x.shape
+    x_flat = x.reshape(B * T, D)
+    if x_flat.dtype != torch.bfloat16:
+        x_flat = x_flat.to(torch.bfloat16)          # the path computes from bf16 activations
+    shared = None
+    if params.get("shared_gate_proj") is not None:
+        shared = dict(gate_proj=params["shared_gate_proj"], up_proj=params["shared_up_proj"],
+                      down_proj=params["shared_down_proj"])
+    out = moe_experts(x_flat, None, top_k=n_experts_per_token,
+                      experts=dict(gate_proj=params["gate_proj"], up_proj=params["up_proj"],
+                                   down_proj=params["down_proj"]),
+                      routing="softmax", shared=shared, gate_weight=params["gate_weight"],
+                      shared_expert_gate_weight=params.get("shared_expert_gate_weight") if shared is not None else None)
+    return out.reshape(B, T, D).to(x.dtype)

@@ -27,7 +27,11 @@ What pins each function (tests/test_oracle.py holds the checks):
                                 shapes; the scaled ones KAT of the reference
                                 (tests/qwen35/test_fp8.py:65-75)
   combine                       per-token Python loop, expert-relabel
-                                invariance, k=1 / zero-weight cases
+                                invariance, k=1 / zero-weight cases; gate = 1
+                                equals no gate, gate = 0 drops the shared rows
+  router_logits / shared_gate   exact small-integer products (any summation
+                                order gives the same value), Python-float
+                                loops, identity weights; sigmoid(0) = 0.5
 
 PARITY UNPINNED (nothing in the reference or in the mathematics fixes the
 bits): the random streams of jax.random, XLA's bf16 rounding order inside
@@ -332,18 +336,55 @@ def expert_swiglu(xq, sx, experts, group_offsets, dtype=np.float64):
     return bf16_round(y.astype(np.float32)), hq, sh
 
 
-def combine(y, weights, inv_perm, shared=None):
-    """out[t] = sum_s w[t,s] * y[inv_perm[t*k+s]] (+ shared[t]); f32 sum in slot
-    order, one bf16 rounding (reference moe.py:90-94 accumulates in bf16; this
-    path keeps f32 until the end)."""
+def combine(y, weights, inv_perm, shared=None, shared_gate=None):
+    """out[t] = sum_s w[t,s] * y[inv_perm[t*k+s]] (+ shared_gate[t] * shared[t]); f32 sum in
+    slot order, one bf16 rounding (reference moe.py:90-94 accumulates in bf16 and moe.py:279
+    rounds the gated shared rows to bf16 before the add of :281; this path keeps f32 until the end)."""
     M, k = weights.shape
     acc = np.zeros((M, y.shape[1]), dtype=np.float32)
     pos = inv_perm.reshape(M, k)
     for s in range(k):
         acc = (acc + (y[pos[:, s]].astype(np.float32) * weights[:, s:s + 1].astype(np.float32))).astype(np.float32)
     if shared is not None:
-        acc = (acc + shared.astype(np.float32)).astype(np.float32)
+        sh = shared.astype(np.float32)
+        if shared_gate is not None:
+            sh = (sh * shared_gate.astype(np.float32)[:, None]).astype(np.float32)
+        acc = (acc + sh).astype(np.float32)
     return bf16_round(acc)
+
+
+# --------------------------------------------------------------------------
+# router in front of the path (moe.py:50 and :278)
+# --------------------------------------------------------------------------
+
+def router_logits(x, gate_weight):
+    """moe.py:50-51: logits = (x @ gate_weight) as a bf16 matmul result, widened to f32.
+    x (M, D) and gate_weight (D, E) hold bf16-representable values.  The sum is taken in
+    float64 (every product of two bf16 values is exact there) and rounded once to f32,
+    then to bf16: the value an f32-accumulating matmul approaches, free of any summation
+    order.  A hardware matmul differs from it by its f32 accumulation error, which shows
+    after the bf16 rounding only for sums that sit on a rounding boundary."""
+    acc = np.asarray(x, np.float64) @ np.asarray(gate_weight, np.float64)
+    return bf16_round(acc.astype(np.float32))
+
+
+def shared_gate(x, shared_expert_gate_weight):
+    """moe.py:278: sigmoid(x @ shared_expert_gate_weight), a bf16 value per token; (M,) f32."""
+    z = router_logits(x, shared_expert_gate_weight)[:, 0]
+    return bf16_round(sigmoid_det(z))
+
+
+def moe_layer(x, params, top_k, dtype=np.float64):
+    """moe.py:235-282 on (M, D) rows: softmax routing on the router's own logits, routed experts,
+    shared expert scaled by its sigmoid gate, one add.  params: gate_weight (D, E); experts / shared
+    dicts as in moe_experts; shared_expert_gate_weight (D, 1) or absent."""
+    logits = router_logits(x, params["gate_weight"])
+    r = moe_experts(x, logits, params["experts"], top_k=top_k, routing="softmax", shared=params.get("shared"),
+                    shared_gate_values=(shared_gate(x, params["shared_expert_gate_weight"])
+                                        if params.get("shared_expert_gate_weight") is not None else None),
+                    dtype=dtype)
+    r["logits"] = logits
+    return r
 
 
 # --------------------------------------------------------------------------
@@ -351,7 +392,8 @@ def combine(y, weights, inv_perm, shared=None):
 # --------------------------------------------------------------------------
 
 def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=None, n_group=1,
-                topk_group=1, renorm=True, routed_scale=1.0, shared=None, dtype=np.float64):
+                topk_group=1, renorm=True, routed_scale=1.0, shared=None, shared_gate_values=None,
+                dtype=np.float64):
     """x: (M,D) float32 holding bf16-representable values.  experts/shared: dicts
     gate/up/down -> (codes, scale_inv) with expert weights (E,N,K) and shared (1,N,K)."""
     E = experts["gate"][0].shape[0]
@@ -369,7 +411,7 @@ def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=Non
     if shared is not None:
         M = x.shape[0]
         ys, _, _ = expert_swiglu(xq, sx, shared, np.array([0, M], dtype=np.int32), dtype=dtype)
-    out = combine(y, w, sg["inv_perm"], ys)
+    out = combine(y, w, sg["inv_perm"], ys, shared_gate_values)
     return dict(out=out, indices=idx, weights=w, xq=xq, sx=sx, y=y, hq=hq, sh=sh, shared_out=ys, **sg)
 
 

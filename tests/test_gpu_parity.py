@@ -311,3 +311,126 @@ def test_graph_replay_matches_eager(jg):
     graph.replay()
     torch.cuda.synchronize()
     assert torch.equal(out, want)
+
+
+# ---- router in front of the path (moe.py:50, :278, :235-282) ------------------------------------
+
+def _bf16_ulp(v):
+    """Spacing of bf16 values in the binade of v (8 significant bits)."""
+    return 2.0 ** (np.floor(np.log2(np.maximum(np.abs(v), 2.0 ** -126))) - 7)
+
+
+def _check_logits(got, want, sum_abs):
+    """Floating-point kernel: the matrix cores add in their own order, so a sum that sits on a bf16
+    rounding boundary may round the other way.  Tolerance: every element within one bf16 ulp of the
+    oracle's order-free value plus the f32 accumulation error (2^-18 of the sum of |products|, which
+    is what counts where a logit cancels to almost nothing), and at most 1 % of the elements off at all."""
+    diff = np.abs(got - want)
+    assert (diff <= np.maximum(_bf16_ulp(want), _bf16_ulp(got)) + 2.0 ** -18 * sum_abs).all(), f"worst {diff.max()} at {np.unravel_index(diff.argmax(), diff.shape)}"
+    frac = float((diff > 0).mean())
+    assert frac < 0.01, f"{frac:.4f} of the logits differ"
+    return frac
+
+
+@pytest.mark.parametrize("M,D,E,gate", [(256, 512, 8, True), (64, 7168, 256, True), (300, 1024, 128, False),
+                                        (1, 128, 40, True), (1000, 256, 1000, False)])
+def test_router_logits_vs_oracle(jg, M, D, E, gate):
+    _say("router logits", M, D, E, gate)
+    rng = H.rng_for(100 + M)
+    x = O.bf16_round(rng.standard_normal((M, D), dtype=np.float32))
+    wr = O.bf16_round(rng.standard_normal((D, E), dtype=np.float32) / np.float32(np.sqrt(D)) * 4)
+    wg = O.bf16_round(rng.standard_normal((D, 1), dtype=np.float32) / np.float32(np.sqrt(D)) * 2)
+    res = jg.router_logits(H.to_bf16_cuda(x), H.to_bf16_cuda(wr), H.to_bf16_cuda(wg) if gate else None)
+    logits = (res[0] if gate else res).cpu().numpy()
+    assert np.array_equal(logits, O.bf16_round(logits))               # bf16-representable values
+    frac = _check_logits(logits, O.router_logits(x, wr), np.abs(x).astype(np.float64) @ np.abs(wr).astype(np.float64))
+    _say(f"   {frac:.5f} of the logits differ by one bf16 ulp")
+    if gate:
+        g = res[1].cpu().numpy()
+        want = O.shared_gate(x, wg)
+        assert (np.abs(g - want) <= 2 * np.maximum(_bf16_ulp(want), _bf16_ulp(g))).all()
+        assert float((g != want).mean()) < 0.03
+    # f32 weights are accepted and rounded to bf16 (the values above are bf16 already: same result)
+    import torch
+    again = jg.router_logits(H.to_bf16_cuda(x), H.to_cuda(wr), H.to_cuda(wg) if gate else None)
+    assert torch.equal(again[0] if gate else again, res[0] if gate else res)
+
+
+def test_moe_routing_matches_reference_semantics(jg):
+    """moe.py:37-55: indices/weights are exactly the softmax top-k of the logits the router produced."""
+    _say("moe_routing")
+    rng = H.rng_for(21)
+    M, D, E, k = 200, 512, 32, 4
+    x = O.bf16_round(rng.standard_normal((M, D), dtype=np.float32))
+    wr = O.bf16_round(rng.standard_normal((D, E), dtype=np.float32) / np.float32(np.sqrt(D)) * 4)
+    xd, wd = H.to_bf16_cuda(x), H.to_bf16_cuda(wr)
+    idx, w = jg.moe_routing(xd, wd, k)
+    logits = jg.router_logits(xd, wd).cpu().numpy()
+    ridx, rw = O.route_softmax_topk(logits, k)
+    assert np.array_equal(idx.cpu().numpy(), ridx)
+    assert np.allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=1e-9)
+    assert np.allclose(w.cpu().numpy().sum(-1), 1.0, atol=1e-5)       # tests/qwen35/test_moe.py:52-60
+
+
+def test_moe_layer_full_parity(jg):
+    """moe.py:235-282 with the reference's parameter names: hidden states in, (B, T, D) out.  Routing is exact
+    as a function of the logits the router kernel produced; the output is compared with the oracle run on
+    those logits and on its own (order-free) shared gate."""
+    import torch
+    _say("moe_layer")
+    B, T, D, E, k, I, SI = 2, 96, 512, 16, 2, 256, 256
+    prob = H.make_problem(M=B * T, D=D, E=E, k=k, I=I, SI=SI, seed=8)
+    rng = H.rng_for(22)
+    wr = O.bf16_round(rng.standard_normal((D, E), dtype=np.float32) / np.float32(np.sqrt(D)) * 4)
+    wg = O.bf16_round(rng.standard_normal((D, 1), dtype=np.float32) / np.float32(np.sqrt(D)) * 2)
+    ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
+    params = dict(gate_weight=H.to_bf16_cuda(wr), gate_proj=ex["gate_proj"], up_proj=ex["up_proj"], down_proj=ex["down_proj"],
+                  shared_gate_proj=sh["gate_proj"], shared_up_proj=sh["up_proj"], shared_down_proj=sh["down_proj"],
+                  shared_expert_gate_weight=H.to_bf16_cuda(wg))
+    x3 = H.to_bf16_cuda(prob["x"]).reshape(B, T, D)
+    out = jg.moe_layer(x3, params, k)
+    assert out.shape == (B, T, D) and out.dtype == torch.bfloat16
+    # the same call through moe_experts exposes the intermediates
+    out2, dbg = jg.moe_experts(x3.reshape(B * T, D), None, top_k=k, experts=ex, shared=sh, gate_weight=params["gate_weight"],
+                               shared_expert_gate_weight=params["shared_expert_gate_weight"], return_debug=True)
+    assert torch.equal(out.reshape(B * T, D), out2)
+    logits = dbg["logits"].cpu().numpy()
+    _check_logits(logits, O.router_logits(prob["x"], wr), np.abs(prob["x"]).astype(np.float64) @ np.abs(wr).astype(np.float64))
+    ref = O.moe_experts(prob["x"], logits, prob["experts"], top_k=k, shared=prob["shared"],
+                        shared_gate_values=O.shared_gate(prob["x"], wg))
+    for name in ("indices", "group_sizes", "sorted_token_ids", "inv_perm"):
+        assert np.array_equal(dbg[name].cpu().numpy(), ref[name]), name
+    err = H.assert_close_out(H.bf16_to_np(out2), ref["out"], tol=1e-2, inner=I)
+    _say("   max-normalised error", err)
+    # the gate matters: without it the output differs
+    no_gate = jg.moe_experts(x3.reshape(B * T, D), None, top_k=k, experts=ex, shared=sh, gate_weight=params["gate_weight"])
+    assert not torch.equal(no_gate, out2)
+    # an f32 input comes back as f32 (moe.py:282 casts to x.dtype)
+    out32 = jg.moe_layer(x3.float(), params, k)
+    assert out32.dtype == torch.float32 and torch.equal(out32, out.float())
+    # one GPU only
+    with pytest.raises(NotImplementedError):
+        jg.moe_layer(x3, params, k, n_devices=8, mesh=object())
+
+
+def test_moe_layer_plain_weights(jg):
+    """Unquantised parameters in the reference's layouts (model.py:98-114: experts (E, in, out), shared (in, out))
+    are quantised to block fp8 on first use and give the same result as the pre-quantised dicts."""
+    import torch
+    _say("moe_layer, plain weights")
+    B, T, D, E, k, I, SI = 1, 64, 256, 4, 2, 128, 128
+    g = torch.Generator(device="cuda"); g.manual_seed(3)
+    def rnd(*s, scale=0.05):
+        return (torch.randn(*s, device="cuda", generator=g) * scale).to(torch.bfloat16)
+    plain = dict(gate_weight=rnd(D, E, scale=0.2), gate_proj=rnd(E, D, I), up_proj=rnd(E, D, I), down_proj=rnd(E, I, D),
+                 shared_gate_proj=rnd(D, SI), shared_up_proj=rnd(D, SI), shared_down_proj=rnd(SI, D),
+                 shared_expert_gate_weight=rnd(D, 1, scale=0.2))
+    quant = dict(plain)
+    for n in ("gate_proj", "up_proj", "down_proj"):
+        quant[n] = jg.quantize_weight_block(plain[n].transpose(1, 2).contiguous())
+    for n in ("shared_gate_proj", "shared_up_proj", "shared_down_proj"):
+        quant[n] = jg.quantize_weight_block(plain[n].t().contiguous())
+    x = rnd(B, T, D, scale=1.0)
+    a = jg.moe_layer(x, plain, k)
+    b = jg.moe_layer(x, quant, k)
+    assert torch.equal(a, b) and torch.isfinite(a.float()).all()

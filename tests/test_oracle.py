@@ -8,6 +8,7 @@ import pytest
 import torch
 
 from oracle import moe_oracle as O
+from tests import helpers as H
 
 
 # ---------------------------------------------------------------- codecs
@@ -342,3 +343,51 @@ def test_oracle_matches_committed_fixture_for_config1():
     got = make_fixtures.build()
     for name in want.files:
         assert np.array_equal(want[name], got[name]), name
+
+
+# ---- router in front of the path --------------------------------------------------------------
+
+def test_router_logits_exact_cases_and_python_loop():
+    """Small integers: every partial sum is exact in f32, so any summation order (and any correct
+    implementation) gives the same bits.  Then a Python-float loop on a tiny random case."""
+    rng = H.rng_for(11)
+    x = rng.integers(-4, 5, size=(6, 128)).astype(np.float32)
+    w = rng.integers(-3, 4, size=(128, 5)).astype(np.float32)
+    want = np.array([[sum(int(x[t, k]) * int(w[k, e]) for k in range(128)) for e in range(5)] for t in range(6)], np.float32)
+    assert np.abs(want).max() < 256                       # representable in bf16
+    assert np.array_equal(O.router_logits(x, w), want)
+    # identity weights copy the activations (already bf16 values)
+    xb = O.bf16_round(rng.standard_normal((4, 128), dtype=np.float32))
+    assert np.array_equal(O.router_logits(xb, np.eye(128, dtype=np.float32)), xb)
+    # transposed-operand mistake fails: (D, E) orientation matters
+    wb = O.bf16_round(rng.standard_normal((128, 128), dtype=np.float32))
+    assert not np.array_equal(O.router_logits(xb, wb), O.router_logits(xb, wb.T.copy()))
+    got = O.router_logits(xb, wb)
+    for t in range(2):
+        for e in range(3):
+            exact = sum(float(xb[t, k]) * float(wb[k, e]) for k in range(128))   # Python floats are f64
+            assert got[t, e] == O.bf16_round(np.array([exact], np.float32))[0]
+
+
+def test_shared_gate_values():
+    x = np.zeros((3, 128), np.float32)
+    w = np.ones((128, 1), np.float32)
+    assert np.array_equal(O.shared_gate(x, w), np.full(3, 0.5, np.float32))            # sigmoid(0)
+    x[1, :4] = 1.0                                                                      # logit 4
+    g = O.shared_gate(x, w)
+    assert abs(float(g[1]) - 1.0 / (1.0 + np.exp(-4.0))) < 2 ** -8                      # bf16 rounding of 0.982
+    assert np.array_equal(g, O.bf16_round(g)) and g[0] == 0.5
+
+
+def test_combine_gate_special_cases():
+    rng = H.rng_for(12)
+    M, k, D = 5, 2, 16
+    y = O.bf16_round(rng.standard_normal((M * k, D), dtype=np.float32))
+    sh = O.bf16_round(rng.standard_normal((M, D), dtype=np.float32))
+    w = rng.random((M, k), dtype=np.float32)
+    inv = rng.permutation(M * k).astype(np.int32)
+    assert np.array_equal(O.combine(y, w, inv, sh, np.ones(M, np.float32)), O.combine(y, w, inv, sh))
+    assert np.array_equal(O.combine(y, w, inv, sh, np.zeros(M, np.float32)), O.combine(y, w, inv))
+    g = np.array([0.5, 0.25, 1.0, 0.0, 0.75], np.float32)
+    want = np.stack([sum(np.float64(w[t, s]) * y[inv[t * k + s]] for s in range(k)) + np.float64(g[t]) * sh[t] for t in range(M)])
+    assert np.abs(O.combine(y, w, inv, sh, g) - want).max() < 0.02
