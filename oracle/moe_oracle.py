@@ -35,7 +35,8 @@ What pins each function (tests/test_oracle.py holds the checks):
 
 PARITY UNPINNED (nothing in the reference or in the mathematics fixes the
 bits): the random streams of jax.random, XLA's bf16 rounding order inside
-ragged_dot and scatter-add, and the case of two distinct logits whose f32
+ragged_dot and scatter-add, XLA's accumulation order inside the router's bf16
+matmul (router_logits takes the order-free value: exact sum, one rounding), and the case of two distinct logits whose f32
 softmax probabilities collide (this oracle ranks logits; the reference ranks
 probabilities, moe.py:51-52).  The reference cannot be imported here (JAX is
 not installed), and it holds no golden vectors for this path.
