@@ -95,10 +95,11 @@ int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
 /* moe.py:90-94 (_scatter_back) as a deterministic gather: out[t] = sum_s w[t,s] *
  * y[inv_perm[t*k+s]] (+ shared_gate[t] * shared[t]) in f32, one bf16 rounding.  shared may be
  * NULL (moe.py:281 adds the shared expert's output); shared_gate may be NULL (= 1; moe.py:278-279
- * multiplies the shared expert's output by sigmoid(x @ shared_expert_gate_weight)). */
+ * multiplies the shared expert's output by sigmoid(x @ shared_expert_gate_weight)); residual
+ * (M, D) bf16 or NULL is the layer's input added last (x = x + moe_out, block.py:58 and :91). */
 int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
-                const void* shared_bf16, const float* shared_gate, int M, int k, int D, void* out_bf16,
-                moe_stream_t stream);
+                const void* shared_bf16, const float* shared_gate, const void* residual_bf16, int M, int k,
+                int D, void* out_bf16, moe_stream_t stream);
 
 /* moe.py:50 (logits = matmul_maybe_fp8(x, gate_weight), a bf16 matmul widened to f32 by :51) and
  * moe.py:278 (sigmoid(x @ shared_expert_gate_weight)).  w_router is (E, D) bf16, K-contiguous (the
@@ -109,6 +110,13 @@ size_t moe_router_workspace_bytes(int M, int D, int E);
 int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
                       const void* w_shared_gate_bf16, float* logits, float* shared_gate, void* ws,
                       size_t ws_bytes, moe_stream_t stream);
+
+/* primitives.py:16-32 (rms_norm, Qwen3.5 convention: x / sqrt(mean(x^2) + eps) * (1 + weight), result in
+ * bf16) as called in front of the MoE layer (block.py:54, :88), fused with the 1x128 quantisation of the
+ * normalised row.  weight (D) f32; normed_bf16 (M, D) may be NULL when only the fp8 form is needed.
+ * D <= 8192. */
+int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
+                      uint8_t* xq, float* sx, moe_stream_t stream);
 
 /* The whole path (moe.py:97-114 + 225-232 + 281): router logits in, combined hidden
  * states out -- or, with w_router set, hidden states in (moe.py:235-282, moe_layer). */
@@ -138,6 +146,10 @@ typedef struct MoeForwardArgs {
   const void* w_shared_gate;     /* (1, D) bf16 or NULL: shared expert's output is scaled by
                                     sigmoid(x . w_shared_gate^T), moe.py:278-279; needs w_router and SI > 0 */
   float* out_logits;             /* (M, E) optional debug output of the computed logits */
+  /* the steps either side of the layer (block.py:54-58, :88-91); NULL / 0 = off */
+  const float* norm_weight;      /* (D) f32: x is RMS-normalised first (rms_norm with 1 + weight, in bf16) */
+  float norm_eps;
+  int add_residual;              /* out = x + moe_out, added in f32 before the one bf16 rounding */
 } MoeForwardArgs;
 
 size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI);

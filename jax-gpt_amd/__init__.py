@@ -15,9 +15,11 @@ from .moe import (  # noqa: F401
     moe_experts,
     moe_layer,
     moe_routing,
+    moe_sublayer,
     permute,
     quant_act,
     quantize_weight_block,
+    rmsnorm_quant,
     route_sigmoid_grouped,
     router_logits,
     route_softmax_topk,

@@ -34,6 +34,7 @@ class MoeForwardArgs(C.Structure):
         ("out_idx", C.c_void_p), ("out_w", C.c_void_p), ("out_group_sizes", C.c_void_p),
         ("out_sorted_token_ids", C.c_void_p), ("out_inv_perm", C.c_void_p),
         ("w_router", C.c_void_p), ("w_shared_gate", C.c_void_p), ("out_logits", C.c_void_p),
+        ("norm_weight", C.c_void_p), ("norm_eps", C.c_float), ("add_residual", C.c_int),
     ]
 
 
@@ -52,7 +53,8 @@ SIGNATURES = {
     "moe_gemm_workspace_bytes": (_Z, [_I, _I, _I]),
     "moe_gemm_gateup_swiglu_fp8": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _Z, _P]),
     "moe_gemm_down_fp8": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _Z, _P]),
-    "moe_combine": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _P, _P]),
+    "moe_combine": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _P]),
+    "moe_rmsnorm_quant": (_I, [_P, _P, _F, _I, _I, _P, _P, _P, _P]),
     "moe_router_workspace_bytes": (_Z, [_I, _I, _I]),
     "moe_router_logits": (_I, [_P, _I, _I, _P, _I, _P, _P, _P, _P, _Z, _P]),
     "moe_forward_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I]),

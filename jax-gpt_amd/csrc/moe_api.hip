@@ -67,7 +67,7 @@ struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
   float *w, *sx, *sh, *shs, *logits, *shared_gate;
   uint8_t *xq, *hq, *hsq;
-  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared, *router_ws;
+  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared, *router_ws, *normed;
   size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, router_ws_bytes, total;
 };
 
@@ -102,10 +102,19 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool r
   b.shared_gate = router ? (float*)c.take((size_t)M * 4) : nullptr;
   b.router_ws_bytes = router ? moe_router_workspace_bytes(M, D, E) : 0;
   b.router_ws = router ? c.take(b.router_ws_bytes) : nullptr;
+  b.normed = router ? c.take((size_t)M * D * 2) : nullptr;   // RMS-normalised activations (norm_weight)
   b.total = c.used;
   return b;
 }
 
+}  // namespace
+
+namespace {
+// the activations the layer computes from: x itself, or its RMS-normalised form (kept in bf16 for the router)
+int quantise(const MoeForwardArgs* a, const ForwardBuffers& b, moe_stream_t stream) {
+  if (a->norm_weight) return moe_rmsnorm_quant(a->x, a->norm_weight, a->norm_eps, a->M, a->D, b.normed, b.xq, b.sx, stream);
+  return moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream);
+}
 }  // namespace
 
 extern "C" size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI) {
@@ -166,7 +175,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
       return moe_check_hip(e, "forward: fork");
     }
     quant_joined = false;
-    rc_shared = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, (moe_stream_t)side);
+    rc_shared = quantise(a, b, (moe_stream_t)side);
     if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
     if (!rc_shared)
@@ -177,7 +186,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
       rc_shared = moe_gemm_down_fp8(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
                                     b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
   } else {
-    if ((rc = moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream))) return rc;
+    if ((rc = quantise(a, b, stream))) return rc;
   }
   // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
   auto join = [&](int code) {
@@ -196,7 +205,13 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   const float* shared_gate = nullptr;
   if (a->w_router) {
     float* lg = a->out_logits ? a->out_logits : b.logits;
-    if ((rc = moe_router_logits(a->x, a->M, a->D, a->w_router, a->E, a->w_shared_gate, lg,
+    // the router reads the normalised activations, which the (possibly forked) quantiser writes
+    if (a->norm_weight && !quant_joined) {
+      if (rc_shared) return join(rc_shared);
+      if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
+      quant_joined = true;
+    }
+    if ((rc = moe_router_logits(a->norm_weight ? b.normed : a->x, a->M, a->D, a->w_router, a->E, a->w_shared_gate, lg,
                                 a->w_shared_gate ? b.shared_gate : nullptr, b.router_ws, b.router_ws_bytes, stream)))
       return join(rc);
     logits = lg;
@@ -225,5 +240,6 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
                                b.gemm_ws_down, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;
-  return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, shared_gate, a->M, a->k, a->D, a->out, stream);
+  return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, shared_gate, a->add_residual ? a->x : nullptr, a->M, a->k,
+                     a->D, a->out, stream);
 }

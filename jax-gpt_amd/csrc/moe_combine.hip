@@ -4,7 +4,8 @@
 // scatter-add) and the final add of moe.py:281.  One workgroup per token; each
 // thread owns 8 consecutive columns, reads its k expert rows through the
 // inverse permutation, sums in f32 in slot order (the shared expert's row last,
-// times its per-token gate of moe.py:278-279 when there is one) and rounds once to bf16.
+// times its per-token gate of moe.py:278-279 when there is one, then the layer's
+// residual input, block.py:58 / :91, when the caller passes it) and rounds once to bf16.
 // HBM-bound: reads k+1 rows, writes one, all as 16-byte accesses.
 #include "moe_common.h"
 
@@ -16,7 +17,8 @@ constexpr int kMaxK = 32;
 __global__ __launch_bounds__(256) void combine_kernel(const bf16x8* __restrict__ y, const float* __restrict__ w,
                                                      const int32_t* __restrict__ inv_perm,
                                                      const bf16x8* __restrict__ shared,
-                                                     const float* __restrict__ shared_gate, int k, int D8,
+                                                     const float* __restrict__ shared_gate,
+                                                     const bf16x8* __restrict__ residual, int k, int D8,
                                                      bf16x8* __restrict__ out) {
   __shared__ int pos[kMaxK];
   __shared__ float wt[kMaxK];
@@ -45,6 +47,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16x8* __restrict__
         for (int i = 0; i < 8; ++i) acc[i] = __fadd_rn(acc[i], bf16_to_f32(v.v[i]));
       }
     }
+    if (residual) {
+      bf16x8 v = residual[(size_t)t * D8 + c];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = __fadd_rn(acc[i], bf16_to_f32(v.v[i]));
+    }
     bf16x8 o;
 #pragma unroll
     for (int i = 0; i < 8; ++i) o.v[i] = f32_to_bf16(acc[i]);
@@ -55,16 +62,17 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16x8* __restrict__
 }  // namespace
 
 extern "C" int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
-                           const void* shared_bf16, const float* shared_gate, int M, int k, int D, void* out_bf16,
-                           moe_stream_t stream) {
+                           const void* shared_bf16, const float* shared_gate, const void* residual_bf16, int M,
+                           int k, int D, void* out_bf16, moe_stream_t stream) {
   MOE_REQUIRE(y_bf16 && w && inv_perm && out_bf16, MOE_ERR_NULL, "combine: null pointer");
   MOE_REQUIRE(M >= 0 && k >= 1 && k <= kMaxK && D > 0 && D % 8 == 0, MOE_ERR_BAD_SHAPE,
               "combine: need 1 <= k <= %d and D %% 8 == 0, got M=%d k=%d D=%d", kMaxK, M, k, D);
-  MOE_REQUIRE(MOE_ALIGNED16(y_bf16) && MOE_ALIGNED16(out_bf16) && MOE_ALIGNED16(shared_bf16), MOE_ERR_BAD_ALIGN,
+  MOE_REQUIRE(MOE_ALIGNED16(y_bf16) && MOE_ALIGNED16(out_bf16) && MOE_ALIGNED16(shared_bf16) &&
+                  MOE_ALIGNED16(residual_bf16), MOE_ERR_BAD_ALIGN,
               "combine: pointers must be 16-byte aligned");
   MOE_REQUIRE(shared_bf16 || !shared_gate, MOE_ERR_NULL, "combine: a shared gate needs a shared expert output");
   if (M == 0) return MOE_OK;
   hipLaunchKernelGGL(combine_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, (const bf16x8*)y_bf16, w, inv_perm,
-                     (const bf16x8*)shared_bf16, shared_gate, k, D / 8, (bf16x8*)out_bf16);
+                     (const bf16x8*)shared_bf16, shared_gate, (const bf16x8*)residual_bf16, k, D / 8, (bf16x8*)out_bf16);
   return moe_check_hip(hipGetLastError(), "combine launch");
 }

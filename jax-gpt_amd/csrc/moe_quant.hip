@@ -37,6 +37,68 @@ __global__ __launch_bounds__(256) void quant_act_kernel(const bf16x8* __restrict
   }
 }
 
+// RMSNorm fused with the activation quantiser: one workgroup per row, the row stays in registers between the
+// two passes.  normed = bf16((x / sqrt(mean(x^2) + eps)) * (1 + weight)), the Qwen3.5 convention of
+// jax_gpt/models/qwen35/primitives.py:16-32 (the step in front of the MoE layer, block.py:54 and :88), then
+// the 1x128 quantisation of the bf16 values.  Thread t holds the 16-byte pieces t, t + 256, ... of the row, so
+// the 16 lanes of a quantisation group are neighbours as in quant_act_kernel.  Sums are taken in a fixed order
+// with individually rounded operations.
+constexpr int kNormPieces = 4;   // D <= 256 * 8 * 4 = 8192
+
+__global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const bf16x8* __restrict__ x, const float* __restrict__ weight,
+                                                           float eps, int D, bf16x8* __restrict__ normed,
+                                                           uint2* __restrict__ xq, float* __restrict__ sx) {
+  __shared__ float wave_sum[4];
+  const int row = blockIdx.x, P = D / 8, t = threadIdx.x;
+  const bf16x8* xr = x + (size_t)row * P;
+  float f[kNormPieces][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kNormPieces; ++i) {
+    const int p = t + 256 * i;
+    bf16x8 in = {};
+    if (p < P) in = xr[p];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      f[i][j] = bf16_to_f32(in.v[j]);
+      ss = __fadd_rn(ss, __fmul_rn(f[i][j], f[i][j]));
+    }
+  }
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) ss = __fadd_rn(ss, __shfl_xor(ss, off, MOE_WAVE));
+  if ((t & 63) == 0) wave_sum[t >> 6] = ss;
+  __syncthreads();
+  const float total = __fadd_rn(__fadd_rn(wave_sum[0], wave_sum[1]), __fadd_rn(wave_sum[2], wave_sum[3]));
+  const float rms = __fsqrt_rn(__fadd_rn(__fdiv_rn(total, (float)D), eps));
+#pragma unroll
+  for (int i = 0; i < kNormPieces; ++i) {
+    const int p = t + 256 * i;
+    const bool ok = p < P;              // uniform over the 16 lanes of a group (P is a multiple of 16)
+    float amax = 0.f;
+    bf16x8 nb = {};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float wj = ok ? weight[p * 8 + j] : 0.f;
+      const float v = __fmul_rn(__fdiv_rn(f[i][j], rms), __fadd_rn(1.0f, wj));
+      nb.v[j] = f32_to_bf16(v);
+      f[i][j] = bf16_to_f32(nb.v[j]);
+      amax = fmaxf(amax, fabsf(f[i][j]));
+    }
+#pragma unroll
+    for (int off = 1; off < 16; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, MOE_WAVE));
+    float scale, scale_inv;
+    fp8_scales(amax, scale, scale_inv);
+    if (ok) {
+      if (normed) normed[(size_t)row * P + p] = nb;
+      uint2 out;
+      out.x = pack4_e4m3(f[i][0] * scale, f[i][1] * scale, f[i][2] * scale, f[i][3] * scale);
+      out.y = pack4_e4m3(f[i][4] * scale, f[i][5] * scale, f[i][6] * scale, f[i][7] * scale);
+      xq[(size_t)row * P + p] = out;
+      if ((t & 15) == 0) sx[((size_t)row * P + p) >> 4] = scale_inv;
+    }
+  }
+}
+
 // one workgroup per 128x128 block; thread t reads row t/2, columns (t%2)*64 .. +64
 template <typename T>
 __global__ __launch_bounds__(256) void quant_weight_kernel(const T* __restrict__ w, int N, int K,
@@ -81,6 +143,19 @@ extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, floa
   hipLaunchKernelGGL(quant_act_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                      (const bf16x8*)x_bf16, pieces, K / 128, (uint2*)xq, sx);
   return moe_check_hip(hipGetLastError(), "quant_act launch");
+}
+
+extern "C" int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
+                                 uint8_t* xq, float* sx, moe_stream_t stream) {
+  MOE_REQUIRE(x_bf16 && weight && xq && sx, MOE_ERR_NULL, "rmsnorm_quant: null pointer");
+  MOE_REQUIRE(M >= 0 && D > 0 && D % MOE_QBLOCK == 0 && D <= 256 * 8 * kNormPieces, MOE_ERR_BAD_SHAPE,
+              "rmsnorm_quant: D=%d must be a multiple of 128, at most %d (M=%d)", D, 256 * 8 * kNormPieces, M);
+  MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(xq) && MOE_ALIGNED16(normed_bf16), MOE_ERR_BAD_ALIGN,
+              "rmsnorm_quant: pointers must be 16-byte aligned");
+  if (M == 0) return MOE_OK;
+  hipLaunchKernelGGL(rmsnorm_quant_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, (const bf16x8*)x_bf16, weight, eps,
+                     D, (bf16x8*)normed_bf16, (uint2*)xq, sx);
+  return moe_check_hip(hipGetLastError(), "rmsnorm_quant launch");
 }
 
 extern "C" int moe_quant_weight_block(const void* w, int src_is_f32, int E, int N, int K, uint8_t* wq,

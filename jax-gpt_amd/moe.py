@@ -121,6 +121,21 @@ def quant_act(x):
     return xq.view(torch.float8_e4m3fn), sx
 
 
+def rmsnorm_quant(x, weight, eps=1e-6):
+    """primitives.py:16-32 (rms_norm with 1 + weight) fused with the 1x128 activation quantiser.
+    x (M, D) bf16, weight (D,) -> (normed (M, D) bf16, codes (M, D) uint8, scale_inv (M, D/128) f32)."""
+    x = _dev(x, torch.bfloat16, "x")
+    weight = _dev(weight.to(torch.float32), torch.float32, "weight")
+    M, D = x.shape
+    if tuple(weight.shape) != (D,):
+        raise ValueError(f"weight: expected ({D},), got {tuple(weight.shape)}")
+    normed = _empty((M, D), torch.bfloat16, x)
+    xq = _empty((M, D), torch.uint8, x)
+    sx = _empty((M, D // 128), torch.float32, x)
+    check(lib().moe_rmsnorm_quant(_ptr(x), _ptr(weight), float(eps), M, D, _ptr(normed), _ptr(xq), _ptr(sx), _stream()))
+    return normed, xq, sx
+
+
 def quantize_weight_block(w):
     """(E, out, in) or (out, in) bf16/f32 -> {'w': float8_e4m3fn, 'scale_inv': f32 (.., out/128, in/128)}.
 
@@ -225,18 +240,20 @@ def gemm_down(hq, sh, down, group_offsets):
     return y
 
 
-def combine(y, weights, inv_perm, shared=None, shared_gate=None):
-    """moe.py:90-94 and the add of :281; `shared_gate` (M,) f32 scales the shared rows (moe.py:278-279)."""
+def combine(y, weights, inv_perm, shared=None, shared_gate=None, residual=None):
+    """moe.py:90-94 and the add of :281; `shared_gate` (M,) f32 scales the shared rows (moe.py:278-279);
+    `residual` (M, D) bf16 is the layer input added last (block.py:58)."""
     y = _dev(y, torch.bfloat16, "y")
     weights = _dev(weights, torch.float32, "weights")
     inv_perm = _dev(inv_perm, torch.int32, "inv_perm")
     shared = None if shared is None else _dev(shared, torch.bfloat16, "shared")
     shared_gate = None if shared_gate is None else _dev(shared_gate, torch.float32, "shared_gate")
+    residual = None if residual is None else _dev(residual, torch.bfloat16, "residual")
     M, k = weights.shape
     D = y.shape[1]
     out = _empty((M, D), torch.bfloat16, y)
-    check(lib().moe_combine(_ptr(y), _ptr(weights), _ptr(inv_perm), _ptr(shared), _ptr(shared_gate), M, k, D,
-                            _ptr(out), _stream()))
+    check(lib().moe_combine(_ptr(y), _ptr(weights), _ptr(inv_perm), _ptr(shared), _ptr(shared_gate), _ptr(residual),
+                            M, k, D, _ptr(out), _stream()))
     return out
 
 
@@ -319,14 +336,15 @@ def moe_routing(x, gate_weight, n_experts_per_token):
 
 def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=None, n_group=1, topk_group=1,
                 renorm=True, routed_scale=1.0, shared=None, return_debug=False, gate_weight=None,
-                shared_expert_gate_weight=None):
+                shared_expert_gate_weight=None, norm_weight=None, norm_eps=1e-6, add_residual=False):
     """Router logits in, combined hidden states out (one C-ABI call, `moe_forward`).
 
     x (M, D) bf16; router_logits (M, E) f32; experts / shared: dicts with keys
     'gate_proj', 'up_proj', 'down_proj' holding block-fp8 dicts (or plain arrays).
     With `gate_weight` (D, E) the call computes the logits itself (moe.py:50; pass
     router_logits=None); `shared_expert_gate_weight` (D, 1) then scales the shared
-    expert's output by its sigmoid gate (moe.py:278-279).
+    expert's output by its sigmoid gate (moe.py:278-279).  `norm_weight` (D,) puts the
+    block's RMSNorm in front (block.py:54) and `add_residual` its `x + moe_out` behind (:58).
     Returns (M, D) bf16, plus a dict of the integer intermediates if return_debug."""
     x = _dev(x, torch.bfloat16, "x")
     wr = wsg = None
@@ -361,7 +379,14 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     a = MoeForwardArgs()
     a.M, a.D, a.E, a.k, a.I = M, D, E, top_k, I
     a.routing, a.n_group, a.topk_group, a.renorm, a.routed_scale = ROUTING[routing], n_group, topk_group, int(renorm), routed_scale
-    keep = [x, logits, wg, sg, wu, su, wd, sd, wr, wsg]
+    nw = None
+    if norm_weight is not None:
+        nw = _dev(norm_weight.to(torch.float32), torch.float32, "norm_weight")
+        if tuple(nw.shape) != (D,):
+            raise ValueError(f"norm_weight: expected ({D},), got {tuple(nw.shape)}")
+        a.norm_weight, a.norm_eps = nw.data_ptr(), float(norm_eps)
+    a.add_residual = int(bool(add_residual))
+    keep = [x, logits, wg, sg, wu, su, wd, sd, wr, wsg, nw]
     a.x = x.data_ptr()
     if logits is not None:
         a.logits = logits.data_ptr()
@@ -408,7 +433,15 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     return (out, dbg) if return_debug else out
 
 
-def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=None):
+def moe_sublayer(x, moe_norm_weight, params, n_experts_per_token, rms_norm_eps=1e-6):
+    """The MoE half of a block, block.py:54-58 and :88-91: x + moe_layer(rms_norm(x, moe_norm), params).
+    The norm is fused with the activation quantiser and the residual add with the combine."""
+    return moe_layer(x, params, n_experts_per_token, _norm_weight=moe_norm_weight, _norm_eps=rms_norm_eps,
+                     _add_residual=True)
+
+
+def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=None, *, _norm_weight=None,
+              _norm_eps=1e-6, _add_residual=False):
     """moe.py:235-282: route + routed experts + gated shared expert, (B, T, D) in and out.
 
     `params` holds the reference's keys (model.py:79-114): gate_weight (D, E); gate_proj, up_proj,
@@ -431,5 +464,6 @@ def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=
                       experts=dict(gate_proj=params["gate_proj"], up_proj=params["up_proj"],
                                    down_proj=params["down_proj"]),
                       routing="softmax", shared=shared, gate_weight=params["gate_weight"],
-                      shared_expert_gate_weight=params.get("shared_expert_gate_weight") if shared is not None else None)
+                      shared_expert_gate_weight=params.get("shared_expert_gate_weight") if shared is not None else None,
+                      norm_weight=_norm_weight, norm_eps=_norm_eps, add_residual=_add_residual)
     return out.reshape(B, T, D).to(x.dtype)

@@ -29,6 +29,8 @@ What pins each function (tests/test_oracle.py holds the checks):
   combine                       per-token Python loop, expert-relabel
                                 invariance, k=1 / zero-weight cases; gate = 1
                                 equals no gate, gate = 0 drops the shared rows
+  rms_norm                      constant rows (closed form), scale invariance,
+                                unit mean square at weight 0, torch CPU f32
   router_logits / shared_gate   exact small-integer products (any summation
                                 order gives the same value), Python-float
                                 loops, identity weights; sigmoid(0) = 0.5
@@ -337,7 +339,7 @@ def expert_swiglu(xq, sx, experts, group_offsets, dtype=np.float64):
     return bf16_round(y.astype(np.float32)), hq, sh
 
 
-def combine(y, weights, inv_perm, shared=None, shared_gate=None):
+def combine(y, weights, inv_perm, shared=None, shared_gate=None, residual=None):
     """out[t] = sum_s w[t,s] * y[inv_perm[t*k+s]] (+ shared_gate[t] * shared[t]); f32 sum in
     slot order, one bf16 rounding (reference moe.py:90-94 accumulates in bf16 and moe.py:279
     rounds the gated shared rows to bf16 before the add of :281; this path keeps f32 until the end)."""
@@ -351,7 +353,19 @@ def combine(y, weights, inv_perm, shared=None, shared_gate=None):
         if shared_gate is not None:
             sh = (sh * shared_gate.astype(np.float32)[:, None]).astype(np.float32)
         acc = (acc + sh).astype(np.float32)
+    if residual is not None:                 # block.py:58: x + moe_out, here inside the one rounding
+        acc = (acc + residual.astype(np.float32)).astype(np.float32)
     return bf16_round(acc)
+
+
+def rms_norm(x, weight, eps=1e-6):
+    """primitives.py:16-32: x / sqrt(mean(x^2) + eps) * (1 + weight) in f32, cast to the input's dtype (bf16
+    here).  The mean is taken in float64 and rounded once (order-free, as router_logits does)."""
+    x32 = np.asarray(x, np.float32)
+    ms = (np.square(x32.astype(np.float64)).mean(axis=-1, keepdims=True)).astype(np.float32)
+    rms = np.sqrt(ms + np.float32(eps)).astype(np.float32)
+    normed = (x32 / rms).astype(np.float32)
+    return bf16_round((normed * (np.float32(1.0) + np.asarray(weight, np.float32))).astype(np.float32))
 
 
 # --------------------------------------------------------------------------
@@ -375,7 +389,15 @@ def shared_gate(x, shared_expert_gate_weight):
     return bf16_round(sigmoid_det(z))
 
 
-def moe_layer(x, params, top_k, dtype=np.float64):
+def moe_sublayer(x, moe_norm_weight, params, top_k, eps=1e-6, dtype=np.float64):
+    """block.py:54-58: x + moe_layer(rms_norm(x, moe_norm), params) on (M, D) rows."""
+    normed = rms_norm(x, moe_norm_weight, eps)
+    r = moe_layer(normed, params, top_k, dtype=dtype, residual=x)
+    r["normed"] = normed
+    return r
+
+
+def moe_layer(x, params, top_k, dtype=np.float64, residual=None):
     """moe.py:235-282 on (M, D) rows: softmax routing on the router's own logits, routed experts,
     shared expert scaled by its sigmoid gate, one add.  params: gate_weight (D, E); experts / shared
     dicts as in moe_experts; shared_expert_gate_weight (D, 1) or absent."""
@@ -383,7 +405,7 @@ def moe_layer(x, params, top_k, dtype=np.float64):
     r = moe_experts(x, logits, params["experts"], top_k=top_k, routing="softmax", shared=params.get("shared"),
                     shared_gate_values=(shared_gate(x, params["shared_expert_gate_weight"])
                                         if params.get("shared_expert_gate_weight") is not None else None),
-                    dtype=dtype)
+                    residual=residual, dtype=dtype)
     r["logits"] = logits
     return r
 
@@ -394,7 +416,7 @@ def moe_layer(x, params, top_k, dtype=np.float64):
 
 def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=None, n_group=1,
                 topk_group=1, renorm=True, routed_scale=1.0, shared=None, shared_gate_values=None,
-                dtype=np.float64):
+                residual=None, dtype=np.float64):
     """x: (M,D) float32 holding bf16-representable values.  experts/shared: dicts
     gate/up/down -> (codes, scale_inv) with expert weights (E,N,K) and shared (1,N,K)."""
     E = experts["gate"][0].shape[0]
@@ -412,7 +434,7 @@ def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=Non
     if shared is not None:
         M = x.shape[0]
         ys, _, _ = expert_swiglu(xq, sx, shared, np.array([0, M], dtype=np.int32), dtype=dtype)
-    out = combine(y, w, sg["inv_perm"], ys, shared_gate_values)
+    out = combine(y, w, sg["inv_perm"], ys, shared_gate_values, residual)
     return dict(out=out, indices=idx, weights=w, xq=xq, sx=sx, y=y, hq=hq, sh=sh, shared_out=ys, **sg)
 
 

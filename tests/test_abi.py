@@ -65,8 +65,9 @@ def test_argument_errors_come_back_as_codes(dll):
     assert dll.moe_permute(one, 4, 2, 8, one, one, one, one, one, one, 0, None) == -3              # workspace too small
     assert dll.moe_gemm_gateup_swiglu_fp8(one, one, None, one, one, one, one, one, 4, 16, 100, 128, one, one, one, 1 << 20, None) == -1
     assert dll.moe_gemm_down_fp8(one, one, one, one, one, 4, 16, 128, 128, one, one, 0, None) == -3
-    assert dll.moe_combine(one, one, one, None, None, 4, 40, 128, one, None) == -1
-    assert dll.moe_combine(one, one, one, None, one, 4, 2, 128, one, None) == -5                   # gate without shared rows
+    assert dll.moe_combine(one, one, one, None, None, None, 4, 40, 128, one, None) == -1
+    assert dll.moe_combine(one, one, one, None, one, None, 4, 2, 128, one, None) == -5             # gate without shared rows
+    assert dll.moe_rmsnorm_quant(one, one, 1e-6, 4, 16384, None, one, one, None) == -1              # D > 8192
     assert dll.moe_router_logits(one, 4, 100, one, 8, None, one, None, one, 1 << 20, None) == -1   # D % 128
     assert dll.moe_router_logits(one, 4, 128, one, 8, one, one, None, one, 1 << 20, None) == -5    # gate weight without output
     assert dll.moe_router_logits(one, 4, 128, one, 8, None, one, None, one, 0, None) == -3

@@ -434,3 +434,66 @@ def test_moe_layer_plain_weights(jg):
     a = jg.moe_layer(x, plain, k)
     b = jg.moe_layer(x, quant, k)
     assert torch.equal(a, b) and torch.isfinite(a.float()).all()
+
+
+# ---- the steps either side of the layer (block.py:54-58) ----------------------------------------
+
+@pytest.mark.parametrize("M,D", [(37, 512), (64, 7168), (3, 128), (9, 8192)])
+def test_rmsnorm_quant_vs_oracle(jg, M, D):
+    """Floating-point kernel (the sum of squares is taken in the kernel's own fixed order): normalised values
+    within one bf16 ulp of the oracle on a few elements and equal elsewhere; the fp8 codes and scales are then
+    exactly the oracle's quantisation OF THE KERNEL'S normalised values."""
+    _say("rmsnorm + quant", M, D)
+    rng = H.rng_for(300 + D)
+    x = O.bf16_round(rng.standard_normal((M, D), dtype=np.float32) * 3)
+    w = (rng.standard_normal(D) * 0.2).astype(np.float32)
+    normed, xq, sx = jg.rmsnorm_quant(H.to_bf16_cuda(x), H.to_cuda(w), 1e-6)
+    got = H.bf16_to_np(normed)
+    want = O.rms_norm(x, w, 1e-6)
+    diff = np.abs(got - want)
+    assert (diff <= np.maximum(_bf16_ulp(want), _bf16_ulp(got))).all()
+    assert float((diff > 0).mean()) < 0.01
+    q_ref, s_ref = O.quant_act_group(got)
+    assert np.array_equal(xq.cpu().numpy(), q_ref)
+    assert np.array_equal(sx.cpu().numpy(), s_ref)
+
+
+def test_moe_sublayer_full_parity(jg):
+    """block.py:54-58: x + moe_layer(rms_norm(x)).  Compared with the oracle fed the kernel's own logits
+    (routing exact), within the output tolerance."""
+    import torch
+    _say("moe_sublayer")
+    B, T, D, E, k, I, SI = 1, 160, 512, 16, 2, 256, 128
+    prob = H.make_problem(M=B * T, D=D, E=E, k=k, I=I, SI=SI, seed=9)
+    rng = H.rng_for(23)
+    x = O.bf16_round(prob["x"] * 2.5)
+    wn = (rng.standard_normal(D) * 0.1).astype(np.float32)
+    wr = O.bf16_round(rng.standard_normal((D, E), dtype=np.float32) / np.float32(np.sqrt(D)) * 4)
+    wg = O.bf16_round(rng.standard_normal((D, 1), dtype=np.float32) / np.float32(np.sqrt(D)) * 2)
+    ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
+    params = dict(gate_weight=H.to_bf16_cuda(wr), gate_proj=ex["gate_proj"], up_proj=ex["up_proj"], down_proj=ex["down_proj"],
+                  shared_gate_proj=sh["gate_proj"], shared_up_proj=sh["up_proj"], shared_down_proj=sh["down_proj"],
+                  shared_expert_gate_weight=H.to_bf16_cuda(wg))
+    xd = H.to_bf16_cuda(x).reshape(B, T, D)
+    out = jg.moe_sublayer(xd, H.to_cuda(wn), params, k, 1e-6)
+    assert out.shape == (B, T, D)
+    out2, dbg = jg.moe_experts(xd.reshape(B * T, D), None, top_k=k, experts=ex, shared=sh, gate_weight=params["gate_weight"],
+                               shared_expert_gate_weight=params["shared_expert_gate_weight"], norm_weight=H.to_cuda(wn),
+                               norm_eps=1e-6, add_residual=True, return_debug=True)
+    assert torch.equal(out.reshape(B * T, D), out2)
+    # the oracle from the kernel's normalised activations and logits on
+    normed = H.bf16_to_np(jg.rmsnorm_quant(xd.reshape(B * T, D), H.to_cuda(wn), 1e-6)[0])
+    want_n = O.rms_norm(x, wn, 1e-6)
+    assert float((normed != want_n).mean()) < 0.01
+    logits = dbg["logits"].cpu().numpy()
+    _check_logits(logits, O.router_logits(normed, wr), np.abs(normed).astype(np.float64) @ np.abs(wr).astype(np.float64))
+    ref = O.moe_experts(normed, logits, prob["experts"], top_k=k, shared=prob["shared"],
+                        shared_gate_values=O.shared_gate(normed, wg), residual=x)
+    for name in ("indices", "group_sizes", "sorted_token_ids", "inv_perm"):
+        assert np.array_equal(dbg[name].cpu().numpy(), ref[name]), name
+    err = H.assert_close_out(H.bf16_to_np(out2), ref["out"], tol=1e-2, inner=I)
+    _say("   max-normalised error", err)
+    # the unfused composition gives the same bits: norm, then the layer, then the residual added in the combine
+    layer = jg.moe_experts(torch.from_numpy(normed).to(torch.bfloat16).cuda(), None, top_k=k, experts=ex, shared=sh,
+                           gate_weight=params["gate_weight"], shared_expert_gate_weight=params["shared_expert_gate_weight"])
+    assert not torch.equal(layer, out2)                      # the residual is in there

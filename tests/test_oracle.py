@@ -391,3 +391,40 @@ def test_combine_gate_special_cases():
     g = np.array([0.5, 0.25, 1.0, 0.0, 0.75], np.float32)
     want = np.stack([sum(np.float64(w[t, s]) * y[inv[t * k + s]] for s in range(k)) + np.float64(g[t]) * sh[t] for t in range(M)])
     assert np.abs(O.combine(y, w, inv, sh, g) - want).max() < 0.02
+
+
+def test_rms_norm_closed_forms():
+    """primitives.py:16-32.  A constant row c gives c / sqrt(c^2 + eps) * (1 + w); scaling the input leaves
+    the output unchanged (up to eps); weight 0 gives unit mean square; and torch's f32 arithmetic agrees."""
+    D = 256
+    w = np.linspace(-0.5, 0.5, D).astype(np.float32)
+    x = np.full((1, D), 3.0, np.float32)
+    want = O.bf16_round((np.float32(3.0) / np.sqrt(np.float32(9.0) + np.float32(1e-6)) * (1 + w)).astype(np.float32))
+    assert np.array_equal(O.rms_norm(x, w, 1e-6)[0], want)
+    rng = H.rng_for(13)
+    xr = O.bf16_round(rng.standard_normal((5, D), dtype=np.float32))
+    a, b = O.rms_norm(xr, w, 1e-12), O.rms_norm(4 * xr, w, 1e-12)            # 4x is exact in bf16
+    assert np.array_equal(a, b)
+    n0 = O.rms_norm(xr, np.zeros(D, np.float32), 0.0)
+    assert np.allclose(np.square(n0.astype(np.float64)).mean(-1), 1.0, atol=4e-3)
+    xt = torch.from_numpy(xr)
+    ref = (xt / torch.sqrt(xt.square().mean(-1, keepdim=True) + 1e-6) * (1 + torch.from_numpy(w))).to(torch.bfloat16).float().numpy()
+    got = O.rms_norm(xr, w, 1e-6)
+    assert float((got != ref).mean()) < 0.01 and np.abs(got - ref).max() <= 2.0 ** -6   # summation order only
+    # a dropped "1 +" or a missing eps would fail these
+    assert not np.array_equal(O.rms_norm(xr, w, 1e-6), O.rms_norm(xr, w - 1, 1e-6))
+    assert np.isfinite(O.rms_norm(np.zeros((1, D), np.float32), w, 1e-6)).all()
+
+
+def test_combine_residual():
+    rng = H.rng_for(14)
+    M, k, D = 4, 2, 8
+    y = O.bf16_round(rng.standard_normal((M * k, D), dtype=np.float32))
+    w = rng.random((M, k), dtype=np.float32)
+    inv = rng.permutation(M * k).astype(np.int32)
+    res = O.bf16_round(rng.standard_normal((M, D), dtype=np.float32))
+    plain = O.combine(y, w, inv)
+    assert np.array_equal(O.combine(y, w, inv, residual=np.zeros((M, D), np.float32)), plain)
+    got = O.combine(y, w, inv, residual=res)
+    want = np.stack([sum(np.float64(w[t, s]) * y[inv[t * k + s]] for s in range(k)) + res[t] for t in range(M)])
+    assert np.abs(got - want).max() < 0.03
