@@ -24,7 +24,10 @@
 // inside the workgroup.  Waves form a 4 x 2 grid: wave (wi, xj) owns weight rows
 // {32wi..32wi+31} of each half (GATEUP) or {64wi..64wi+63} (DOWN) against the
 // 16-row activation fragments 2j + xj (alternating between the two wave sets, so
-// a short tile still splits evenly).  Two tile heights are built:
+// a short tile still splits evenly).  Three tile heights are built:
+//   BM = 32:  wave tile 64 x 16, two stages of 36 KB, TWO workgroups per CU: for batches of a few rows per
+//             expert the kernel only streams weights, and a second workgroup keeps the stream going while
+//             the first starts or finishes a work item;
 //   BM = 128: wave tile 64 x 64, three stages of 48.5 KB (copies two steps ahead);
 //   BM = 256: wave tile 64 x 128, two stages of 65 KB (copies one, twice as long,
 //             step ahead); half the weight traffic, LDS reads and barriers per MFMA.
@@ -147,10 +150,11 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
 constexpr int MAX_KB = 256;   // K <= 32768
 constexpr int W_TILE_BYTES = BW * BK;   // 32 KB
 
-template <int XW>   // XW = 1: BM = 128, XW = 2: BM = 256
+template <int XW>   // XW = 0: BM = 32 (two workgroups per CU), XW = 1: BM = 128, XW = 2: BM = 256
 struct Cfg {
-  static constexpr int BM = 128 * XW;
-  static constexpr int XF = 4 * XW;                            // activation fragments per wave
+  static constexpr int BM = XW == 0 ? 32 : 128 * XW;
+  static constexpr int XF = BM / 32;                           // activation fragments per wave
+  static constexpr int WG_PER_CU = XW == 0 ? 2 : 1;
   static constexpr int NSTAGE = XW == 1 ? 3 : 2;
   static constexpr int PRE = NSTAGE - 1;                       // copies run PRE steps ahead
   static constexpr int X_TILE_BYTES = BM * BK;
@@ -160,8 +164,9 @@ struct Cfg {
   static constexpr int WSCALE_OFF = NSTAGE * STAGE_BYTES;      // [2][MAX_KB] weight block scales of the work item
   static constexpr int RING_BYTES = WSCALE_OFF + 2 * MAX_KB * 4;
   static constexpr int EPI_BYTES = BM * 512;                   // bf16 staging of MODE_DOWN (<= RING_BYTES)
-  static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // 151040 / 133120
-  static constexpr int X_DMA = 2 * XW;                         // 1 KB activation row groups per wave per step
+  static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // 76032 / 151040 / 133120
+  static constexpr int X_DMA = XW == 0 ? 1 : 2 * XW;           // 1 KB activation row groups per wave per step
+                                                               // (at BM = 32 only waves 0-3 have one: see XSKIP)
   static constexpr int VM_PER_STEP = 4 + X_DMA + 1;            // + 4 weight row groups + 1 scale copy
   // skip the copies of activation rows past the end of a short tile; only where every step waits for all of its
   // copies anyway (PRE == 1), so that no wait has to count a varying number of them
@@ -174,7 +179,7 @@ struct Cfg {
 #ifndef MOE_ROT2
 #define MOE_ROT2 1
 #endif
-  static constexpr int ROT = XW == 1 ? MOE_ROT1 : MOE_ROT2;
+  static constexpr int ROT = XW == 0 ? 0 : XW == 1 ? MOE_ROT1 : MOE_ROT2;
 };
 
 // Sched<XW>::first(j) = index of the first copy operation issued after MFMA group j (first(XF) = VM_PER_STEP).
@@ -187,10 +192,11 @@ template <int XW> struct Sched {
   static constexpr int first(int j) {
     constexpr int n = Cfg<XW>::VM_PER_STEP, g = Cfg<XW>::XF;
     if (j >= g) return n;
+    if (j <= 0) return 0;
     if (MOE_SCHED == 1) return (n * j) / g;                    // even
-    if (MOE_SCHED == 2) { int h = g / 2; return j >= h ? n : (n * j) / h; }   // all in the first half of the step
-    if (MOE_SCHED == 3) { int h = (3 * g) / 4; return j >= h ? n : (n * j) / h; }
-    return j == 0 ? 0 : n;
+    if (MOE_SCHED == 2) { int h = g / 2 > 0 ? g / 2 : 1; return j >= h ? n : (n * j) / h; }   // first half of the step
+    if (MOE_SCHED == 3) { int h = (3 * g) / 4 > 0 ? (3 * g) / 4 : 1; return j >= h ? n : (n * j) / h; }
+    return n;
   }
 };
 
@@ -217,7 +223,7 @@ template <int N> __device__ __forceinline__ void wait_vm() {
 }
 
 template <int MODE, int XW>
-__global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
+__global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0,   // gate (GATEUP) or down (DOWN)
     const uint8_t* __restrict__ w1, const float* __restrict__ sw1,   // up (GATEUP only)
@@ -392,8 +398,13 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
       float sxv[XF];
 #pragma unroll
       for (int j = 0; j < XF; j += 4) {
-        const v4f a = *(const v4f*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + j * 4);
-        sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
+        if constexpr (XF >= 4) {
+          const v4f a = *(const v4f*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + j * 4);
+          sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
+        } else {
+#pragma unroll
+          for (int q = 0; q < XF; ++q) sxv[q] = *(const float*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + q * 4);
+        }
       }
       v8i xf[XA + 1];
 #pragma unroll
@@ -481,7 +492,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     __syncthreads();
     const int ld_chunk = tid & 7, ld_row = tid >> 3;   // 64 rows per pass
 #pragma unroll
-    for (int i = 0; i < BM / 64; ++i) {
+    for (int i = 0; i < (BM + 63) / 64; ++i) {
       const int r = ld_row + 64 * i;
       if (r < item.row_count) {
         v4i v = *(const v4i*)(tile + swz(r, ld_chunk));
@@ -552,17 +563,22 @@ int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const
   return moe_check_hip(hipGetLastError(), "gemm launch");
 }
 
-// MOE_GEMM_BM=128|256 in the environment pins the tile height for experiments; default: by shape
+// MOE_GEMM_BM=32|128|256 in the environment pins the tile height for experiments; default: by shape
 int forced_xw() {
   static int v = [] {
     const char* e = getenv("MOE_GEMM_BM");
     return e ? atoi(e) : 0;
   }();
-  return v == 128 ? 1 : v == 256 ? 2 : 0;
+  return v == 32 ? 0 : v == 128 ? 1 : v == 256 ? 2 : -1;
 }
 
-// 256-row tiles once the average expert has more than 128 rows, 128-row tiles otherwise
-int tile_config(int R, int E) { return forced_xw() ? forced_xw() : ((long long)R > 128ll * E ? 2 : 1); }
+// 256-row tiles once the average expert has more than 128 rows, 32-row tiles (two workgroups per CU: one streams
+// weights while the other starts or finishes an item) when it has at most 16, 128-row tiles between
+int tile_config(int R, int E) {
+  if (forced_xw() >= 0) return forced_xw();
+  return (long long)R > 128ll * E ? 2 : (long long)R <= 16ll * E ? 0 : 1;
+}
+int tile_height(int cfg) { return cfg == 0 ? 32 : 128 * cfg; }
 
 template <int MODE>
 int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
@@ -574,8 +590,12 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
   MOE_REQUIRE((long long)N * K <= (1ll << 32) && (long long)R * K <= (1ll << 32), MOE_ERR_BAD_SHAPE,
               "gemm: one expert matrix and the activation array must each stay within 4 GB (N=%d K=%d R=%d)", N, K, R);
   if (R == 0) return MOE_OK;
-  if (tile_config(R, E) == 2)
+  const int cfg = tile_config(R, E);
+  if (cfg == 2)
     return launch_cfg<MODE, 2>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
+                               list_built, s);
+  if (cfg == 0)
+    return launch_cfg<MODE, 0>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
                                list_built, s);
   return launch_cfg<MODE, 1>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
                              list_built, s);
@@ -584,9 +604,10 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
 }  // namespace
 
 extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
-  // enough for either GEMM and either tile height: column blocks of 128 and 128-row tiles bound every case
+  // enough for either GEMM: column blocks of 128 bound both; the tile height is the one the launch will choose
   int ncb = (N_out + 127) / 128;
-  return sizeof(WorkHeader) + (size_t)max_items_for(R, E, ncb, 128) * sizeof(WorkItem) + 256;
+  const int bm = tile_height(tile_config(R, E));
+  return sizeof(WorkHeader) + (size_t)max_items_for(R, E, ncb, bm < 128 ? bm : 128) * sizeof(WorkItem) + 256;
 }
 
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
@@ -637,7 +658,7 @@ int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int 
   MOE_REQUIRE(ws_bytes_each >= moe_gemm_workspace_bytes(R, E, I > D ? I : D), MOE_ERR_WORKSPACE_TOO_SMALL,
               "gemm lists: workspace too small");
   if (R == 0) return MOE_OK;
-  const int bm = tile_config(R, E) == 2 ? 256 : 128;
+  const int bm = tile_height(tile_config(R, E));
   const int ncb_a = col_blocks(MODE_GATEUP, I), ncb_b = col_blocks(MODE_DOWN, D);
   const ListSpec a{ncb_a, max_items_for(R, E, ncb_a, bm), (WorkHeader*)ws_gateup,
                    (WorkItem*)((char*)ws_gateup + sizeof(WorkHeader))};
