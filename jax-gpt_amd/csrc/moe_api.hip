@@ -128,7 +128,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
               "forward: bad dims M=%d D=%d E=%d k=%d I=%d SI=%d", a->M, a->D, a->E, a->k, a->I, a->SI);
   MOE_REQUIRE(a->D % 128 == 0 && a->I % 128 == 0 && a->SI % 128 == 0, MOE_ERR_BAD_SHAPE,
               "forward: D=%d, I=%d and SI=%d must be multiples of 128", a->D, a->I, a->SI);
-  MOE_REQUIRE(a->x && (a->logits || a->w_router) && a->out && a->w_gate && a->w_up && a->w_down && a->sw_gate && a->sw_up && a->sw_down,
+  MOE_REQUIRE((a->M == 0 || (a->x && (a->logits || a->w_router) && a->out)) && a->w_gate && a->w_up && a->w_down && a->sw_gate && a->sw_up && a->sw_down,
               MOE_ERR_NULL, "forward: null tensor pointer");
   if (a->SI)
     MOE_REQUIRE(a->ws_gate && a->ws_up && a->ws_down && a->sws_gate && a->sws_up && a->sws_down, MOE_ERR_NULL,

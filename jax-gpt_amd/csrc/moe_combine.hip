@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16x8* __restrict__
 extern "C" int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
                            const void* shared_bf16, const float* shared_gate, const void* residual_bf16, int M,
                            int k, int D, void* out_bf16, moe_stream_t stream) {
-  MOE_REQUIRE(y_bf16 && w && inv_perm && out_bf16, MOE_ERR_NULL, "combine: null pointer");
+  MOE_REQUIRE(M == 0 || (y_bf16 && w && inv_perm && out_bf16), MOE_ERR_NULL, "combine: null pointer");
   MOE_REQUIRE(M >= 0 && k >= 1 && k <= kMaxK && D > 0 && D % 8 == 0, MOE_ERR_BAD_SHAPE,
               "combine: need 1 <= k <= %d and D %% 8 == 0, got M=%d k=%d D=%d", kMaxK, M, k, D);
   MOE_REQUIRE(MOE_ALIGNED16(y_bf16) && MOE_ALIGNED16(out_bf16) && MOE_ALIGNED16(shared_bf16) &&

@@ -614,7 +614,7 @@ int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_
                          const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
                          int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,
                          moe_stream_t stream) {
-  MOE_REQUIRE(xq && sx && w_gate && sw_gate && w_up && sw_up && group_offsets && hq && sh && ws, MOE_ERR_NULL,
+  MOE_REQUIRE((R == 0 || (xq && sx && hq && sh)) && w_gate && sw_gate && w_up && sw_up && group_offsets && ws, MOE_ERR_NULL,
               "gemm_gateup: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0 && D > 0 && I > 0 && D % 128 == 0 && I % 128 == 0, MOE_ERR_BAD_SHAPE,
               "gemm_gateup: need D %% 128 == 0 and I %% 128 == 0 and 1 <= E <= 1024, got E=%d R=%d D=%d I=%d", E, R, D, I);
@@ -636,7 +636,8 @@ extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, co
 int moe_gemm_down_impl(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
                        const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
                        size_t ws_bytes, bool list_built, moe_stream_t stream) {
-  MOE_REQUIRE(hq && sh && w_down && sw_down && group_offsets && y_bf16 && ws, MOE_ERR_NULL, "gemm_down: null pointer");
+  MOE_REQUIRE((R == 0 || (hq && sh && y_bf16)) && w_down && sw_down && group_offsets && ws, MOE_ERR_NULL,
+              "gemm_down: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0 && D > 0 && I > 0 && D % 128 == 0 && I % 128 == 0, MOE_ERR_BAD_SHAPE,
               "gemm_down: need D %% 128 == 0 and I %% 128 == 0 and 1 <= E <= 1024, got E=%d R=%d I=%d D=%d", E, R, I, D);
   MOE_REQUIRE(MOE_ALIGNED16(hq) && MOE_ALIGNED16(w_down) && MOE_ALIGNED16(y_bf16) && MOE_ALIGNED16(ws), MOE_ERR_BAD_ALIGN,

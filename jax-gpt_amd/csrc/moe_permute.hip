@@ -223,7 +223,7 @@ extern "C" size_t moe_permute_workspace_bytes(int M, int k, int E) {
 extern "C" int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* group_sizes,
                            int32_t* group_offsets, int32_t* sorted_token_ids, int32_t* sort_order,
                            int32_t* inv_perm, void* ws, size_t ws_bytes, moe_stream_t stream) {
-  MOE_REQUIRE(idx && group_sizes && group_offsets && ws, MOE_ERR_NULL, "permute: null pointer");
+  MOE_REQUIRE((idx || M == 0) && group_sizes && group_offsets && ws, MOE_ERR_NULL, "permute: null pointer");
   MOE_REQUIRE(M >= 0 && k >= 1 && E >= 1 && E <= kMaxE, MOE_ERR_BAD_SHAPE,
               "permute: need k >= 1 and 1 <= E <= %d, got M=%d k=%d E=%d", kMaxE, M, k, E);
   MOE_REQUIRE((long long)M * k < (1ll << 31), MOE_ERR_BAD_SHAPE, "permute: M*k overflows int32");

@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256) void quant_weight_kernel(const T* __restrict__
 }  // namespace
 
 extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream) {
-  MOE_REQUIRE(x_bf16 && xq && sx, MOE_ERR_NULL, "quant_act: null pointer");
+  MOE_REQUIRE(R == 0 || (x_bf16 && xq && sx), MOE_ERR_NULL, "quant_act: null pointer");
   MOE_REQUIRE(R >= 0 && K > 0 && K % MOE_QBLOCK == 0, MOE_ERR_BAD_SHAPE, "quant_act: K=%d must be a positive multiple of 128 (R=%d)", K, R);
   MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(xq), MOE_ERR_BAD_ALIGN, "quant_act: pointers must be 16-byte aligned");
   if (R == 0) return MOE_OK;
@@ -147,7 +147,7 @@ extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, floa
 
 extern "C" int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
                                  uint8_t* xq, float* sx, moe_stream_t stream) {
-  MOE_REQUIRE(x_bf16 && weight && xq && sx, MOE_ERR_NULL, "rmsnorm_quant: null pointer");
+  MOE_REQUIRE((M == 0 || (x_bf16 && xq && sx)) && weight, MOE_ERR_NULL, "rmsnorm_quant: null pointer");
   MOE_REQUIRE(M >= 0 && D > 0 && D % MOE_QBLOCK == 0 && D <= 256 * 8 * kNormPieces, MOE_ERR_BAD_SHAPE,
               "rmsnorm_quant: D=%d must be a multiple of 128, at most %d (M=%d)", D, 256 * 8 * kNormPieces, M);
   MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(xq) && MOE_ALIGNED16(normed_bf16), MOE_ERR_BAD_ALIGN,

@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
 }
 
 int check_route_args(const float* logits, int M, int E, int k, const int32_t* idx, const float* w) {
-  MOE_REQUIRE(logits && idx && w, MOE_ERR_NULL, "route: null pointer");
+  MOE_REQUIRE(M == 0 || (logits && idx && w), MOE_ERR_NULL, "route: null pointer");
   MOE_REQUIRE(M >= 0 && E >= 1 && E <= 1024, MOE_ERR_BAD_SHAPE, "route: need 1 <= E <= 1024, got E=%d M=%d", E, M);
   MOE_REQUIRE(k >= 1 && k <= 32 && k <= E, MOE_ERR_BAD_SHAPE, "route: need 1 <= k <= min(32,E), got k=%d E=%d", k, E);
   return MOE_OK;

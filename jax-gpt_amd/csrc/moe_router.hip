@@ -87,7 +87,8 @@ __global__ __launch_bounds__(256) void router_finish_kernel(const float* __restr
 }
 
 int choose_splits(int M, int N, int D) {
-  const long long tiles = (long long)((M + RT - 1) / RT) * ((N + RN - 1) / RN);
+  long long tiles = (long long)((M + RT - 1) / RT) * ((N + RN - 1) / RN);
+  if (tiles < 1) tiles = 1;                  // M = 0
   long long s = (512 + tiles - 1) / tiles;   // aim for about two workgroups per CU
   const int max_s = D / 128;
   if (s > max_s) s = max_s;
@@ -106,7 +107,7 @@ extern "C" size_t moe_router_workspace_bytes(int M, int D, int E) {
 extern "C" int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
                                  const void* w_shared_gate_bf16, float* logits, float* shared_gate, void* ws,
                                  size_t ws_bytes, moe_stream_t stream) {
-  MOE_REQUIRE(x_bf16 && w_router_bf16 && logits && ws, MOE_ERR_NULL, "router: null pointer");
+  MOE_REQUIRE((M == 0 || (x_bf16 && logits)) && w_router_bf16 && ws, MOE_ERR_NULL, "router: null pointer");
   MOE_REQUIRE((w_shared_gate_bf16 == nullptr) == (shared_gate == nullptr), MOE_ERR_NULL,
               "router: the shared gate's weight and output come together");
   MOE_REQUIRE(M >= 0 && D > 0 && D % 128 == 0 && E >= 1 && E <= 1024, MOE_ERR_BAD_SHAPE,

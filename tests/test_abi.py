@@ -78,6 +78,9 @@ def test_workspace_sizes_are_monotone(dll):
     a = dll.moe_forward_workspace_bytes(64, 7168, 256, 8, 2048, 2048)
     b = dll.moe_forward_workspace_bytes(8192, 7168, 256, 8, 2048, 2048)
     assert 0 < a < b < 4 << 30
+    assert dll.moe_forward_workspace_bytes(0, 7168, 256, 8, 2048, 2048) > 0          # an empty batch sizes a workspace too
+    assert dll.moe_router_workspace_bytes(0, 7168, 256) >= 0
+    assert dll.moe_router_workspace_bytes(8192, 7168, 256) >= 8192 * 257 * 4
     assert dll.moe_permute_workspace_bytes(8192, 8, 256) >= 32 * 256 * 4
     assert dll.moe_gemm_workspace_bytes(65536, 256, 7168) > dll.moe_gemm_workspace_bytes(512, 256, 7168) > 0
 

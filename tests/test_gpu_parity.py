@@ -499,3 +499,31 @@ def test_moe_sublayer_full_parity(jg):
     layer = jg.moe_experts(torch.from_numpy(normed).to(torch.bfloat16).cuda(), None, top_k=k, experts=ex, shared=sh,
                            gate_weight=params["gate_weight"], shared_expert_gate_weight=params["shared_expert_gate_weight"])
     assert not torch.equal(layer, out2)                      # the residual is in there
+
+
+def test_empty_batch_and_limits(jg):
+    """M = 0 goes through every entry point without a launch; E = 1024 / k = 32 are the documented maxima."""
+    import torch
+    _say("empty batch, maxima")
+    prob = H.make_problem(M=4, D=128, E=4, k=2, I=128, SI=128, seed=40)
+    ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
+    x0 = torch.empty((0, 128), dtype=torch.bfloat16, device="cuda")
+    lg0 = torch.empty((0, 4), dtype=torch.float32, device="cuda")
+    out = jg.moe_experts(x0, lg0, top_k=2, experts=ex, shared=sh)
+    assert out.shape == (0, 128)
+    idx, w = jg.route_softmax_topk(lg0, 2)
+    assert idx.shape == (0, 2)
+    sg = jg.permute(idx, 4)
+    assert sg["group_sizes"].cpu().tolist() == [0, 0, 0, 0] and sg["group_offsets"].cpu().tolist() == [0] * 5
+    # the widest router the kernels take: 1024 experts, top-32
+    rng = H.rng_for(41)
+    logits = rng.standard_normal((33, 1024), dtype=np.float32)
+    idx, w = jg.route_softmax_topk(H.to_cuda(logits), 32)
+    ridx, rw = O.route_softmax_topk(logits, 32)
+    assert np.array_equal(idx.cpu().numpy(), ridx) and np.allclose(w.cpu().numpy(), rw, rtol=2e-6, atol=1e-9)
+    sg = jg.permute(idx, 1024)
+    rsg = O.sort_and_group(ridx, 1024)
+    for name in ("group_sizes", "group_offsets", "sorted_token_ids", "inv_perm"):
+        assert np.array_equal(sg[name].cpu().numpy(), rsg[name]), name
+    with pytest.raises(jg.MoeError):
+        jg.route_softmax_topk(H.to_cuda(rng.standard_normal((2, 1025), dtype=np.float32)), 2)
