@@ -23,7 +23,7 @@ COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-
           "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 # routing and combine promise individually rounded f32 operations (bit-reproducible on a CPU)
 PER_FILE = {"moe_route.hip": ["-ffp-contract=off"], "moe_combine.hip": ["-ffp-contract=off"],
-            "moe_router.hip": ["-ffp-contract=off"],
+            "moe_router.hip": ["-ffp-contract=off", "-Wno-inline-asm"],
             # MFMA results go straight to VGPRs: the block-scale FMA consumes them on the vector ALU
             "moe_gemm.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-Wno-inline-asm"]}   # m0 is clobbered on purpose
 

@@ -203,25 +203,6 @@ template <int XW> struct Sched {
 // epilogue staging tile: 128-byte rows, chunk c of row r at position c ^ (r & 7)
 __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 4); }
 
-// The copies are inline assembly on purpose: when the compiler knows that an instruction writes LDS from
-// memory it makes every later LDS read wait for ALL outstanding memory operations, which would empty the
-// prefetch queue at every K step.  Completion is tracked by hand instead (wait_vm + barrier); these are the
-// only vector-memory operations inside the K loop.  The LDS destination of lane l is m0 + l * size; the
-// source address is a uniform 64-bit base (scalar registers) + a per-lane 32-bit byte offset.
-__device__ __forceinline__ void dma16(const uint8_t* base, unsigned off, uint8_t* l) {
-  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
-}
-__device__ __forceinline__ void dma4(const uint8_t* base, unsigned off, uint8_t* l) {
-  const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
-}
-__device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(0xC07F); }   // lgkmcnt = 0, other counters untouched
-template <int N> __device__ __forceinline__ void wait_vm() {
-  static_assert(N >= 0 && N < 64, "vmcnt range");
-  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));   // vmcnt = N, other counters untouched
-}
-
 template <int MODE, int XW>
 __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,

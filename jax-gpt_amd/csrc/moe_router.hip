@@ -17,57 +17,99 @@ namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 
-constexpr int RT = 64;    // tokens per workgroup
-constexpr int RN = 256;   // output columns per workgroup (64 per wave)
-constexpr int RK = 32;    // K per MFMA
+constexpr int RT = 128;   // tokens per workgroup
+constexpr int RN = 128;   // output columns per workgroup
+constexpr int RBK = 64;   // K elements per step = one 128-byte LDS row
+constexpr int R_TILE = RT * RBK * 2;            // 16 KB per operand tile
+constexpr int R_STAGE = 2 * R_TILE;             // activations + weights
+constexpr int R_LDS = 2 * R_STAGE;              // two stages: two workgroups fit one CU
 
-// Wave tile 64 tokens x 64 columns = 4 x 4 MFMA tiles of 16 x 16.  Lane (fr = lane % 16, fq = lane / 16)
-// supplies K elements [8 fq, 8 fq + 8) of row fr for both operands, straight from global memory (16 bytes per
-// lane; x and w rows are re-read through L1/L2 by the waves that share them).  Output register r of a tile is
-// (token 4 fq + r, column fr).
-__global__ __launch_bounds__(256) void router_gemm_kernel(const bf16_t* __restrict__ x, int M, int D,
-                                                         const bf16_t* __restrict__ w, int E,
-                                                         const bf16_t* __restrict__ w_extra, int N, int k_per_split,
-                                                         float* __restrict__ partial) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// Workgroup = 4 waves in a 2 x 2 grid, wave tile 64 tokens x 64 columns = 4 x 4 MFMA tiles of 16 x 16 (K = 32 per
+// v_mfma_f32_16x16x32_bf16, two per step).  Both operand tiles go global -> LDS without registers in between
+// (global_load_lds_dwordx4: a wave instruction fills 8 rows of 128 bytes), two stages, copies one step ahead,
+// completion counted by hand.  LDS rows are 128 bytes; the 16-byte chunk c of row r sits at position
+// c ^ ((r >> 1) & 7), which makes the fragment reads (row = lane % 16, chunk = 4 s + lane / 16) conflict-free.
+// Lane (fr = lane % 16, fq = lane / 16) supplies K elements [32 s + 8 fq, +8) of row fr for both operands;
+// output register r of a tile is (token 4 fq + r, column fr).  Weight rows take a full address per lane: the
+// shared gate's row lives in its own allocation.
+__global__ __launch_bounds__(256, 2) void router_gemm_kernel(const bf16_t* __restrict__ x, int M, int D,
+                                                            const bf16_t* __restrict__ w, int E,
+                                                            const bf16_t* __restrict__ w_extra, int N, int k_per_split,
+                                                            float* __restrict__ partial) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
   const int fr = lane & 15, fq = lane >> 4;
-  const int t0 = blockIdx.x * RT, n0 = blockIdx.y * RN + wave * 64;
-  if (n0 >= N) return;   // uniform per wave
+  const int t0 = blockIdx.x * RT, n0 = blockIdx.y * RN;
   const int k0 = blockIdx.z * k_per_split, k1 = min(D, k0 + k_per_split);
-  const bf16_t* xa[4];
-  const bf16_t* wb[4];
+  const int steps = (k1 - k0) / RBK;
+
+  // copy sources: wave v fills row groups [4v, 4v + 4) (8 rows each) of both tiles
+  const int drow = lane >> 3, dchunk = lane & 7;
+  unsigned xoff[4];
+  const bf16_t* wsrc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    xa[i] = x + (size_t)min(t0 + 16 * i + fr, M - 1) * D + fq * 8;
-    const int n = min(n0 + 16 * i + fr, N - 1);
-    wb[i] = (n < E ? w + (size_t)n * D : w_extra) + fq * 8;
+    const int r = (wave * 4 + i) * 8 + drow;
+    const int piece = dchunk ^ ((r >> 1) & 7);
+    xoff[i] = (unsigned)min(t0 + r, M - 1) * (unsigned)D * 2u + piece * 16;   // M * D * 2 < 4 GB (checked by the launcher)
+    const int n = min(n0 + r, N - 1);
+    wsrc[i] = (n < E ? w + (size_t)n * D : w_extra) + piece * 8 + k0;
   }
+  auto issue = [&](int s) {   // 8 operations
+    uint8_t* st = lds + (s & 1) * R_STAGE;
+    const uint8_t* xk = (const uint8_t*)(x + k0 + (size_t)s * RBK);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16(xk, xoff[i], st + (wave * 4 + i) * 1024);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) dma16_addr(wsrc[i] + (size_t)s * RBK, st + R_TILE + (wave * 4 + i) * 1024);
+  };
   v4f acc[4][4];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = (v4f){0.f, 0.f, 0.f, 0.f};
-  for (int k = k0; k < k1; k += RK) {
-    bf16x8_t a[4], b[4];
+  // column fragments past the last column are never multiplied (uniform per wave)
+  const int jmax = min(4, max(0, (N - n0 - wn * 64 + 15) >> 4));
+
+  if (steps > 0) issue(0);
+  for (int s = 0; s < steps; ++s) {
+    wait_vm<0>();                     // this wave's copies of stage s have landed
+    __builtin_amdgcn_s_barrier();     // ... and everyone's; stage s - 1 is free again
+    if (s + 1 < steps) issue(s + 1);
+    const uint8_t* st = lds + (s & 1) * R_STAGE;
+    const uint8_t* xa = st + (wm * 64 + fr) * 128;
+    const uint8_t* wb = st + R_TILE + (wn * 64 + fr) * 128;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      a[i] = *(const bf16x8_t*)(xa[i] + k);
-      b[i] = *(const bf16x8_t*)(wb[i] + k);
+    for (int h = 0; h < 2; ++h) {
+      const int pos = ((4 * h + fq) ^ (fr >> 1)) << 4;
+      bf16x8_t a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a[i] = __builtin_bit_cast(bf16x8_t, *(const v4i*)(xa + i * 16 * 128 + pos));
+        b[i] = __builtin_bit_cast(bf16x8_t, *(const v4i*)(wb + i * 16 * 128 + pos));
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (j < jmax) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+      }
     }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    wait_lgkm0();   // this wave's reads of stage s are done before anyone overwrites it (after the next barrier)
   }
   float* out = partial + (size_t)blockIdx.z * M * N;
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int n = n0 + 16 * j + fr;
+      const int n = n0 + wn * 64 + 16 * j + fr;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int t = t0 + 16 * i + 4 * fq + r;
+        const int t = t0 + wm * 64 + 16 * i + 4 * fq + r;
         if (t < M && n < N) out[(size_t)t * N + n] = acc[i][j][r];
       }
     }
@@ -120,11 +162,18 @@ extern "C" int moe_router_logits(const void* x_bf16, int M, int D, const void* w
   if (M == 0) return MOE_OK;
   const int N = E + (w_shared_gate_bf16 ? 1 : 0);
   const int splits = choose_splits(M, N, D);
-  const int k_per_split = ((D / RK + splits - 1) / splits) * RK;
+  const int k_per_split = ((D / RBK + splits - 1) / splits) * RBK;
   const int used = (D + k_per_split - 1) / k_per_split;   // slices that hold at least one K step
+  MOE_REQUIRE((long long)M * D * 2 < (1ll << 32), MOE_ERR_BAD_SHAPE, "router: the activations must stay within 4 GB");
   float* partial = (float*)ws;
   hipStream_t s = (hipStream_t)stream;
-  hipLaunchKernelGGL(router_gemm_kernel, dim3((M + RT - 1) / RT, (N + RN - 1) / RN, used), dim3(256), 0, s,
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t err = hipFuncSetAttribute((const void*)router_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, R_LDS);
+    if (err != hipSuccess) return moe_check_hip(err, "router: raising the dynamic LDS limit");
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(router_gemm_kernel, dim3((M + RT - 1) / RT, (N + RN - 1) / RN, used), dim3(256), R_LDS, s,
                      (const bf16_t*)x_bf16, M, D, (const bf16_t*)w_router_bf16, E, (const bf16_t*)w_shared_gate_bf16, N,
                      k_per_split, partial);
   const long long total = (long long)M * N;
