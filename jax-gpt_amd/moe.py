@@ -156,6 +156,20 @@ def quantize_weight_block(w):
     return {"w": wq.view(torch.float8_e4m3fn), "scale_inv": sw}
 
 
+def block_fp8_from_per_row(d):
+    """The reference's own fp8 dicts carry one scale per output row (`scale_inv` (E, out, 1) or (out, 1),
+    quantize.py:18-42).  This path computes with 128x128 blocks: de-quantise (w * scale_inv, moe.py:29) to f32
+    and quantise again per block.  A second rounding of the weights, so prefer quantising from bf16 where the
+    original weights exist."""
+    q, s = d["w"], d["scale_inv"]
+    if q.dtype != torch.float8_e4m3fn:
+        q = _codes(q, "w").view(torch.float8_e4m3fn)
+    if s.shape[-1] != 1 or s.shape[:-1] != q.shape[:-1]:
+        raise ValueError(f"expected per-row scales {tuple(q.shape[:-1]) + (1,)}, got {tuple(s.shape)}")
+    w = _dev(q, None, "w").to(torch.float32) * _dev(s, None, "scale_inv").to(torch.float32)
+    return quantize_weight_block(w)
+
+
 _plain_cache = {}
 
 
@@ -170,8 +184,8 @@ def _expert_weight(w, name):
         if tuple(s.shape) != (E, N // 128, K // 128):
             raise ValueError(
                 f"{name}: scale_inv has shape {tuple(s.shape)}; this path needs 128x128 block scales "
-                f"{(E, N // 128, K // 128)} (per-row scales of the reference's quantize.py must be re-quantised "
-                "with quantize_weight_block)")
+                f"{(E, N // 128, K // 128)} (per-row scales of the reference's quantize.py must be re-quantised: "
+                "block_fp8_from_per_row(d), or quantize_weight_block on the bf16 weights)")
         return _codes(q, name + "['w']"), _dev(s, torch.float32, name + "['scale_inv']")
     if not isinstance(w, torch.Tensor):
         raise TypeError(f"{name}: expected a tensor or an fp8 dict")

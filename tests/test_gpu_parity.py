@@ -527,3 +527,28 @@ def test_empty_batch_and_limits(jg):
         assert np.array_equal(sg[name].cpu().numpy(), rsg[name]), name
     with pytest.raises(jg.MoeError):
         jg.route_softmax_topk(H.to_cuda(rng.standard_normal((2, 1025), dtype=np.float32)), 2)
+
+
+def test_per_row_fp8_dicts_are_converted_on_request(jg):
+    """The reference's fp8 format (one scale per output row, quantize.py:18-42) is refused by the GEMMs with a
+    message and converted by block_fp8_from_per_row: de-quantise as moe.py:29 does, quantise per 128 x 128 block."""
+    import torch
+    _say("per-row fp8 dicts")
+    E, N, K = 2, 128, 256
+    g = torch.Generator(device="cuda"); g.manual_seed(7)
+    w = torch.randn(E, N, K, device="cuda", generator=g) * 0.05
+    amax = w.abs().amax(dim=-1, keepdim=True)
+    scale_inv = (amax / 448.0).float()                                     # quantize.py:31-42
+    q = (w / scale_inv).clamp(-448, 448).to(torch.float8_e4m3fn)
+    d = {"w": q, "scale_inv": scale_inv}
+    off = torch.tensor([0, 8, 16], dtype=torch.int32, device="cuda")
+    xq, sx = jg.quant_act(torch.randn(16, K, device="cuda", generator=g).to(torch.bfloat16))
+    with pytest.raises(ValueError, match="block_fp8_from_per_row"):
+        jg.gemm_gateup_swiglu(xq, sx, d, d, off)
+    b = jg.block_fp8_from_per_row(d)
+    assert b["w"].shape == (E, N, K) and b["scale_inv"].shape == (E, 1, 2)
+    deq_row = q.float() * scale_inv
+    deq_blk = b["w"].float() * b["scale_inv"].repeat_interleave(128, 1).repeat_interleave(128, 2)
+    assert (deq_blk - deq_row).abs().max() <= 0.07 * deq_row.abs().max()    # one more e4m3 rounding
+    hq, sh = jg.gemm_gateup_swiglu(xq, sx, b, b, off)
+    assert hq.shape == (16, N) and torch.isfinite(sh).all()
