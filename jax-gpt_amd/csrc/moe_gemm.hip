@@ -172,31 +172,36 @@ struct Cfg {
   // copies anyway (PRE == 1), so that no wait has to count a varying number of them
   static constexpr bool XSKIP = PRE == 1;
   // MFMA groups by which wave set 1 trails wave set 0 (build-time tuning knobs; measured best: half a step at
-  // BM = 128, one group at BM = 256 where registers are short)
+  // BM = 128, two of the eight groups at BM = 256, where registers allow no more)
 #ifndef MOE_ROT1
 #define MOE_ROT1 2
 #endif
 #ifndef MOE_ROT2
-#define MOE_ROT2 1
+#define MOE_ROT2 2
 #endif
   static constexpr int ROT = XW == 0 ? 0 : XW == 1 ? MOE_ROT1 : MOE_ROT2;
 };
 
 // Sched<XW>::first(j) = index of the first copy operation issued after MFMA group j (first(XF) = VM_PER_STEP).
-// MOE_SCHED (build-time tuning knob): 0 = all copies at the start of the step, 1 = spread evenly, 2 / 3 = spread
-// over the first half / three quarters of the step (3 measured best).
-#ifndef MOE_SCHED
-#define MOE_SCHED 3
+// The copies of a step are spread over its first XF * NUM / 4 groups (build-time tuning knobs MOE_SCHED1 /
+// MOE_SCHED2 = NUM for BM = 128 / 256; 0 = all copies at the start of the step, 4 = spread over the whole step).
+// Measured best: three quarters of the step at BM = 128 (copies run two steps ahead there), the first half at
+// BM = 256 (one step ahead: the later a copy is issued, the less time it has to land).
+#ifndef MOE_SCHED1
+#define MOE_SCHED1 3
+#endif
+#ifndef MOE_SCHED2
+#define MOE_SCHED2 2
 #endif
 template <int XW> struct Sched {
   static constexpr int first(int j) {
     constexpr int n = Cfg<XW>::VM_PER_STEP, g = Cfg<XW>::XF;
+    constexpr int num = XW == 2 ? MOE_SCHED2 : MOE_SCHED1;
+    constexpr int h = (g * num) / 4 > 0 ? (g * num) / 4 : 1;   // groups that carry copies
     if (j >= g) return n;
     if (j <= 0) return 0;
-    if (MOE_SCHED == 1) return (n * j) / g;                    // even
-    if (MOE_SCHED == 2) { int h = g / 2 > 0 ? g / 2 : 1; return j >= h ? n : (n * j) / h; }   // first half of the step
-    if (MOE_SCHED == 3) { int h = (3 * g) / 4 > 0 ? (3 * g) / 4 : 1; return j >= h ? n : (n * j) / h; }
-    return n;
+    if (num == 0) return n;
+    return j >= h ? n : (n * j) / h;
   }
 };
 
