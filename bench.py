@@ -27,7 +27,7 @@ PEAK_FP8_TFLOPS = 5000.0     # MI355X dense fp8 MFMA (published)
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E (published)
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
 # file (counter x calibration factor; the summary and the commands are in profiles/).  None = not measured.
-MEASURED_TRAFFIC = {"deepseek_v3_prefill": 8536e6 + 143e6}
+MEASURED_TRAFFIC = {"deepseek_v3_prefill": 8757e6 + 146e6}
 
 WORKLOADS = {
     # BASELINE config 3 / 4: DeepSeek-V3-style layer
