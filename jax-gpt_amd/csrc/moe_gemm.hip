@@ -252,7 +252,7 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
   unsigned xoff[C::X_DMA];
 #pragma unroll
   for (int i = 0; i < C::X_DMA; ++i) {
-    const int r = (wave * C::X_DMA + i) * 8 + drow;            // row within the activation tile
+    const int r = (i * NWAVES + wave) * 8 + drow;              // row within the activation tile (groups dealt round-robin)
     const int piece = dchunk ^ ((r >> 1) & 7);
     int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
@@ -271,16 +271,17 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
     soff = (unsigned)g * (unsigned)KB * 4u;
   }
   // With XSKIP, activation row groups that lie wholly past the item's last row are not copied (their LDS rows
-  // keep stale bytes; whatever the matrix cores make of them lands in rows the epilogue never stores).  The valid
-  // groups of a wave are a prefix of its X_DMA groups.
-  const int nxv = C::XSKIP ? min(C::X_DMA, max(0, ((item.row_count + 7) >> 3) - wave * C::X_DMA)) : C::X_DMA;
+  // keep stale bytes; whatever the matrix cores make of them lands in rows the epilogue never stores).  Row group g
+  // (8 rows) belongs to wave g % 8, so the groups of a short tile spread over all the waves and a wave's valid
+  // groups are a prefix of its X_DMA groups.
+  const int nxv = C::XSKIP ? min(C::X_DMA, max(0, (((item.row_count + 7) >> 3) - wave + NWAVES - 1) / NWAVES)) : C::X_DMA;
   // copy operation i (0 <= i < VM_PER_STEP) of K step kb
   auto issue_op = [&](int kb, int i) {
     uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
     if (i < 4) dma16(wmat + (size_t)kb * BK, woff[i], st + (wave * 4 + i) * 1024);
     else if (i < 4 + C::X_DMA) {
       if (!C::XSKIP || i - 4 < nxv)
-        dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + (wave * C::X_DMA + i - 4) * 1024);
+        dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + ((i - 4) * NWAVES + wave) * 1024);
     }
     else if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4);
   };
