@@ -38,8 +38,8 @@ What pins each function (tests/test_oracle.py holds the checks):
 PARITY UNPINNED (nothing in the reference or in the mathematics fixes the
 bits): the random streams of jax.random, XLA's bf16 rounding order inside
 ragged_dot and scatter-add, XLA's accumulation order inside the router's bf16
-matmul (router_logits takes the order-free value: exact sum, one rounding), and the case of two distinct logits whose f32
-softmax probabilities collide (this oracle ranks logits; the reference ranks
+matmul (router_logits takes the order-free value: exact sum, one rounding),
+and the case of two distinct logits whose f32 softmax probabilities collide (this oracle ranks logits; the reference ranks
 probabilities, moe.py:51-52).  The reference cannot be imported here (JAX is
 not installed), and it holds no golden vectors for this path.
 """
@@ -438,10 +438,12 @@ def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=Non
     return dict(out=out, indices=idx, weights=w, xq=xq, sx=sx, y=y, hq=hq, sh=sh, shared_out=ys, **sg)
 
 
-def moe_experts_rows(x, tokens, indices, weights, fetch_expert, shared=None, dtype=np.float64):
+def moe_experts_rows(x, tokens, indices, weights, fetch_expert, shared=None, dtype=np.float64, shared_gate_values=None,
+                     residual=None):
     """The same mathematics for a handful of token rows at full problem size:
     `fetch_expert(e)` returns dict gate/up/down -> (codes (N,K), scale_inv) for
-    expert e.  Returns (len(tokens), D) f32 (bf16-representable)."""
+    expert e.  shared_gate_values (M,) and residual (M, D) as in combine.
+    Returns (len(tokens), D) f32 (bf16-representable)."""
     outs = []
     for t in tokens:
         xq, sx = quant_act_group(x[t:t + 1])
@@ -454,6 +456,10 @@ def moe_experts_rows(x, tokens, indices, weights, fetch_expert, shared=None, dty
             acc = (acc + y * np.float32(weights[t, s])).astype(np.float32)
         if shared is not None:
             ys, _, _ = expert_swiglu(xq, sx, shared, off, dtype=dtype)
+            if shared_gate_values is not None:
+                ys = (ys * np.float32(shared_gate_values[t])).astype(np.float32)
             acc = (acc + ys).astype(np.float32)
+        if residual is not None:
+            acc = (acc + residual[t:t + 1].astype(np.float32)).astype(np.float32)
         outs.append(bf16_round(acc)[0])
     return np.stack(outs)

@@ -175,3 +175,53 @@ def test_config5_expert_parallel_shard_skewed(env):
     toks = [0, 1, M - 1] + list(rng.integers(0, M, 5))
     want_out = O.combine(yn, weights, inv_perm)[toks]
     assert np.array_equal(H.bf16_to_np(out)[toks], want_out)
+
+
+def test_config3_sized_moe_sublayer(env, dsv3_layer):
+    """The rows either side of the path at the benchmark's full size: RMSNorm + router (256 experts, hidden 7168)
+    + softmax top-8 routing + gated shared expert + residual, 8192 tokens.  Router logits and normalised rows are
+    checked on sampled tokens against the oracle; routing is exact as a function of the kernel's logits; sampled
+    output rows against the oracle's per-row path."""
+    jg, torch, bench = env
+    _say("config 3 sized moe_sublayer (norm + router + gate + residual)")
+    cfg = bench.WORKLOADS["deepseek_v3_prefill"]
+    experts, shared, _, _ = dsv3_layer
+    M, D, E, k, I = cfg["M"], cfg["D"], cfg["E"], cfg["k"], cfg["I"]
+    gen = torch.Generator(device="cuda"); gen.manual_seed(50)
+    x = (torch.randn((M, D), dtype=torch.float32, device="cuda", generator=gen) * 2).to(torch.bfloat16)
+    wr = (torch.randn((D, E), dtype=torch.float32, device="cuda", generator=gen) * (4 / D ** 0.5)).to(torch.bfloat16)
+    wg = (torch.randn((D, 1), dtype=torch.float32, device="cuda", generator=gen) * (2 / D ** 0.5)).to(torch.bfloat16)
+    wn = torch.randn((D,), dtype=torch.float32, device="cuda", generator=gen) * 0.1
+    out, dbg = jg.moe_experts(x, None, top_k=k, experts=experts, shared=shared, gate_weight=wr, shared_expert_gate_weight=wg,
+                              norm_weight=wn, norm_eps=1e-6, add_residual=True, return_debug=True)
+    torch.cuda.synchronize()
+    outn = H.bf16_to_np(out)
+    assert np.isfinite(outn).all()
+    rng = H.rng_for(51)
+    tokens = sorted(set([0, M - 1] + list(rng.integers(0, M, 2))))
+    tsel = torch.tensor(tokens, device="cuda")
+    xs = H.bf16_to_np(x[tsel])
+    wrn, wgn, wnn = H.bf16_to_np(wr), H.bf16_to_np(wg), wn.cpu().numpy()
+    # normalised rows and logits of the sampled tokens
+    normed_gpu = H.bf16_to_np(jg.rmsnorm_quant(x[tsel].contiguous(), wn, 1e-6)[0])
+    normed = O.rms_norm(xs, wnn, 1e-6)
+    assert float((normed_gpu != normed).mean()) < 0.01
+    logits = dbg["logits"].cpu().numpy()
+    want_l = O.router_logits(normed_gpu, wrn)
+    got_l = logits[tokens]
+    assert float((got_l != want_l).mean()) < 0.02 and np.abs(got_l - want_l).max() <= 2.0 ** -4
+    # routing: exact as a function of the kernel's own logits, for every token
+    ridx, rw = O.route_softmax_topk(logits, k)
+    assert np.array_equal(dbg["indices"].cpu().numpy(), ridx)
+    sg = O.sort_and_group(ridx, E)
+    assert np.array_equal(dbg["group_sizes"].cpu().numpy(), sg["group_sizes"])
+    assert np.array_equal(dbg["inv_perm"].cpu().numpy(), sg["inv_perm"])
+    # sampled output rows
+    f = _fetch(shared)(0)
+    sh = {n: (q[None], s[None]) for n, (q, s) in f.items()}
+    nfull = np.zeros((max(tokens) + 1, D), np.float32); nfull[tokens] = normed_gpu
+    xfull = np.zeros_like(nfull); xfull[tokens] = xs
+    gate = np.zeros(max(tokens) + 1, np.float32); gate[tokens] = O.shared_gate(normed_gpu, wgn)
+    want = O.moe_experts_rows(nfull, tokens, ridx, rw, _fetch(experts), shared=sh, shared_gate_values=gate, residual=xfull)
+    err = H.assert_close_out(outn[tokens], want, tol=1e-2, inner=I)
+    _say(f"   {len(tokens)} sampled rows: max-normalised error {err:.2e}")
