@@ -28,7 +28,10 @@ __global__ __launch_bounds__(256) void combine_kernel(const bf16x8* __restrict__
     wt[threadIdx.x] = w[(size_t)t * k + threadIdx.x];
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < D8; c += 256) {
+  // gridDim.y workgroups share a token's columns (small batches: one workgroup per token would leave the chip idle)
+  const int per = (D8 + gridDim.y - 1) / gridDim.y;
+  const int c_end = min(D8, (int)(blockIdx.y + 1) * per);
+  for (int c = blockIdx.y * per + threadIdx.x; c < c_end; c += 256) {
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int s = 0; s < k; ++s) {
       bf16x8 v = y[(size_t)pos[s] * D8 + c];
@@ -72,7 +75,10 @@ extern "C" int moe_combine(const void* y_bf16, const float* w, const int32_t* in
               "combine: pointers must be 16-byte aligned");
   MOE_REQUIRE(shared_bf16 || !shared_gate, MOE_ERR_NULL, "combine: a shared gate needs a shared expert output");
   if (M == 0) return MOE_OK;
-  hipLaunchKernelGGL(combine_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, (const bf16x8*)y_bf16, w, inv_perm,
+  // about four workgroups per CU at least: split the columns of a token when there are few tokens
+  int split = 1;
+  while (split < 8 && (long long)M * split < 1024 && (D / 8) / (split * 2) >= 64) split *= 2;
+  hipLaunchKernelGGL(combine_kernel, dim3(M, split), dim3(256), 0, (hipStream_t)stream, (const bf16x8*)y_bf16, w, inv_perm,
                      (const bf16x8*)shared_bf16, shared_gate, (const bf16x8*)residual_bf16, k, D / 8, (bf16x8*)out_bf16);
   return moe_check_hip(hipGetLastError(), "combine launch");
 }

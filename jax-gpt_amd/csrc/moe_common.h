@@ -18,6 +18,54 @@ typedef unsigned short bf16_t;  // raw bf16 bits
 int moe_set_error(int code, const char* fmt, ...);
 int moe_check_hip(hipError_t e, const char* what);
 
+// ---- work list of the grouped GEMMs ----
+struct WorkHeader {
+  int n_items;
+  int pad[3];
+};
+struct WorkItem {
+  int expert, row_start, row_count, col_block;
+};
+struct ListSpec {
+  int n_col_blocks, max_items;   // n_col_blocks == 0: no list wanted
+  WorkHeader* hdr;
+  WorkItem* items;
+};
+// An expert with `rows` rows gets ceil(rows / bm) row tiles of equal height (a multiple of 16, the last one
+// shorter): tiles that share a weight slab then take the same time per K step and walk it together, so the
+// second reader finds it in L2.
+// (integer division costs some forty instructions on this hardware: the one-tile case takes none)
+__host__ __device__ inline int moe_tile_rows(int rows, int bm) {
+  if (rows <= bm) return bm;
+  const int t = (rows + bm - 1) / bm;
+  return ((rows + t - 1) / t + 15) & ~15;
+}
+__host__ __device__ inline int moe_tile_count(int rows, int bm) {
+  if (rows <= 0) return 0;
+  if (rows <= bm) return 1;
+  const int tr = moe_tile_rows(rows, bm);
+  return (rows + tr - 1) / tr;
+}
+// the items of one expert, [col_block][row tile] from position tile_base * n_col_blocks on; `first` / `step` let a
+// group of threads share the expert
+__device__ inline void moe_write_expert_items(const ListSpec& spec, int expert, int row_start, int rows, int tile_base,
+                                              int bm, int first, int step) {
+  const int tiles = moe_tile_count(rows, bm);
+  const int tr = moe_tile_rows(rows, bm);
+  const int n = tiles * spec.n_col_blocks;
+  for (int local = first; local < n; local += step) {
+    const int it = tile_base * spec.n_col_blocks + local;
+    if (it >= spec.max_items) break;   // cannot happen for consistent offsets; keeps writes in bounds
+    const int cb = tiles == 1 ? local : local / tiles, rt = tiles == 1 ? 0 : local - cb * tiles;
+    WorkItem w;
+    w.expert = expert;
+    w.row_start = row_start + rt * tr;
+    w.row_count = min(tr, rows - rt * tr);
+    w.col_block = cb;
+    spec.items[it] = w;
+  }
+}
+
 // grouped GEMMs with an optional pre-built work list (moe_gemm.hip); the extern "C" entry points build their own
 int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
                          size_t ws_bytes_each, moe_stream_t stream);

@@ -56,47 +56,21 @@ constexpr int NT = 64 * NWAVES;
 constexpr int MODE_GATEUP = 0;
 constexpr int MODE_DOWN = 1;
 
-struct WorkHeader {
-  int n_items;
-  int pad[3];
-};
-struct WorkItem {
-  int expert, row_start, row_count, col_block;
-};
-
 // ---- work list -----------------------------------------------------------
 
-// One workgroup.  An expert with rows_e rows gets ceil(rows_e / bm) row tiles of equal height (a multiple of 16,
-// the last one shorter): tiles that share a weight slab then take the same time per K step and walk it together,
-// so the second reader finds it in L2.  Item order [expert][col_block][row tile].
-__device__ __forceinline__ int tile_rows(int rows, int bm) {
-  const int t = (rows + bm - 1) / bm;
-  return t <= 1 ? bm : (((rows + t - 1) / t + 15) & ~15);
-}
-struct ListSpec {
-  int n_col_blocks, max_items;
-  WorkHeader* hdr;
-  WorkItem* items;
-};
-// workgroup b builds list b (the gate/up and the down GEMM of one layer walk the same rows with different
-// column-block counts: one launch lists both)
+// Workgroup b builds list b (the gate/up and the down GEMM of one layer walk the same rows with different
+// column-block counts: one launch lists both).  Item order [expert][col_block][row tile]; each wave writes the
+// items of the experts it owns.
 __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __restrict__ group_offsets, int E, int bm,
                                                           ListSpec l0, ListSpec l1) {
   const ListSpec spec = blockIdx.x == 0 ? l0 : l1;
-  const int n_col_blocks = spec.n_col_blocks, max_items = spec.max_items;
-  WorkHeader* __restrict__ hdr = spec.hdr;
-  WorkItem* __restrict__ items = spec.items;
   __shared__ int tile_prefix[1025];
   __shared__ int wave_tot[16];
   const int e = threadIdx.x;
   const int lane = e & 63, wv = e >> 6;
   int rows = 0;
   if (e < E) rows = group_offsets[e + 1] - group_offsets[e];
-  int tiles = 0;
-  if (rows > 0) {
-    const int tr = tile_rows(rows, bm);
-    tiles = (rows + tr - 1) / tr;
-  }
+  const int tiles = moe_tile_count(rows, bm);
   int incl = tiles;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -110,28 +84,12 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
   if (e < E) tile_prefix[e + 1] = wbase + incl;
   if (e == 0) tile_prefix[0] = 0;
   __syncthreads();
-  int total = tile_prefix[E] * n_col_blocks;
-  if (total > max_items) total = max_items;  // cannot happen for consistent offsets; keeps writes in bounds
-  if (e == 0) hdr->n_items = total;
-  for (int it = threadIdx.x; it < total; it += blockDim.x) {
-    // find expert x with tile_prefix[x]*ncb <= it < tile_prefix[x+1]*ncb
-    int lo = 0, hi = E;
-    while (hi - lo > 1) {
-      int mid = (lo + hi) >> 1;
-      if (tile_prefix[mid] * n_col_blocks <= it) lo = mid; else hi = mid;
-    }
-    const int x = lo;
-    const int tiles_x = tile_prefix[x + 1] - tile_prefix[x];
-    const int local = it - tile_prefix[x] * n_col_blocks;
-    const int cb = local / tiles_x, rt = local % tiles_x;
+  int total = tile_prefix[E] * spec.n_col_blocks;
+  if (total > spec.max_items) total = spec.max_items;
+  if (e == 0) spec.hdr->n_items = total;
+  for (int x = wv; x < E; x += 16) {
     const int start = group_offsets[x], rows_x = group_offsets[x + 1] - start;
-    const int tr = tile_rows(rows_x, bm);
-    WorkItem w;
-    w.expert = x;
-    w.row_start = start + rt * tr;
-    w.row_count = min(tr, rows_x - rt * tr);
-    w.col_block = cb;
-    items[it] = w;
+    if (rows_x > 0) moe_write_expert_items(spec, x, start, rows_x, tile_prefix[x], bm, lane, MOE_WAVE);
   }
 }
 
@@ -639,19 +597,31 @@ extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8
   return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, stream);
 }
 
+namespace {
+int list_specs(int E, int R, int D, int I, void* ws_gateup, void* ws_down, size_t ws_bytes_each, ListSpec* l0,
+               ListSpec* l1, int* bm_out) {
+  MOE_REQUIRE(ws_bytes_each >= moe_gemm_workspace_bytes(R, E, I > D ? I : D), MOE_ERR_WORKSPACE_TOO_SMALL,
+              "gemm lists: workspace too small");
+  const int bm = tile_height(tile_config(R, E));
+  const int ncb_a = col_blocks(MODE_GATEUP, I), ncb_b = col_blocks(MODE_DOWN, D);
+  *l0 = ListSpec{ncb_a, max_items_for(R, E, ncb_a, bm), (WorkHeader*)ws_gateup,
+                 (WorkItem*)((char*)ws_gateup + sizeof(WorkHeader))};
+  *l1 = ListSpec{ncb_b, max_items_for(R, E, ncb_b, bm), (WorkHeader*)ws_down,
+                 (WorkItem*)((char*)ws_down + sizeof(WorkHeader))};
+  *bm_out = bm;
+  return MOE_OK;
+}
+}  // namespace
+
 // Lists the work items of a layer's gate/up GEMM (into ws_gateup) and down GEMM (into ws_down) in one launch;
 // the *_impl entry points then take list_built = true.
 int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
                          size_t ws_bytes_each, moe_stream_t stream) {
-  MOE_REQUIRE(ws_bytes_each >= moe_gemm_workspace_bytes(R, E, I > D ? I : D), MOE_ERR_WORKSPACE_TOO_SMALL,
-              "gemm lists: workspace too small");
+  ListSpec a, b;
+  int bm;
+  int rc = list_specs(E, R, D, I, ws_gateup, ws_down, ws_bytes_each, &a, &b, &bm);
+  if (rc) return rc;
   if (R == 0) return MOE_OK;
-  const int bm = tile_height(tile_config(R, E));
-  const int ncb_a = col_blocks(MODE_GATEUP, I), ncb_b = col_blocks(MODE_DOWN, D);
-  const ListSpec a{ncb_a, max_items_for(R, E, ncb_a, bm), (WorkHeader*)ws_gateup,
-                   (WorkItem*)((char*)ws_gateup + sizeof(WorkHeader))};
-  const ListSpec b{ncb_b, max_items_for(R, E, ncb_b, bm), (WorkHeader*)ws_down,
-                   (WorkItem*)((char*)ws_down + sizeof(WorkHeader))};
   hipLaunchKernelGGL(build_items_kernel, dim3(2), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, bm, a, b);
   return moe_check_hip(hipGetLastError(), "gemm lists launch");
 }
