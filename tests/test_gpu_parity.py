@@ -552,3 +552,30 @@ def test_per_row_fp8_dicts_are_converted_on_request(jg):
     assert (deq_blk - deq_row).abs().max() <= 0.07 * deq_row.abs().max()    # one more e4m3 rounding
     hq, sh = jg.gemm_gateup_swiglu(xq, sx, b, b, off)
     assert hq.shape == (16, N) and torch.isfinite(sh).all()
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_grouped_gemms_random_group_sizes(jg, seed):
+    """Random ragged groups (empty, tiny, just under / over a tile boundary, several tiles) through all three tile
+    heights: every row against the oracle."""
+    rng = H.rng_for(700 + seed)
+    E = int(rng.integers(1, 9))
+    D, I = [(256, 256), (384, 128), (128, 512)][seed % 3]
+    choices = [0, 1, 15, 16, 17, 31, 32, 33, 127, 128, 129, 145, 255, 256, 257, 300, 511, 513]
+    sizes = [int(rng.choice(choices)) for _ in range(E)]
+    if seed % 2:                                   # every other case small enough on average for the 32-row tiles
+        sizes = [min(s, 40) for s in sizes]
+    if sum(sizes) == 0:
+        sizes[0] = 3
+    _say("grouped_gemm random", E, D, I, sizes)
+    off, xq, sx, ex = _ragged_case(800 + seed, E, D, I, sizes)
+    dex = H.experts_to_cuda(ex)
+    hq, sh = jg.gemm_gateup_swiglu(H.to_cuda(xq), H.to_cuda(sx), dex["gate_proj"], dex["up_proj"], H.to_cuda(off))
+    g = O.grouped_gemm(xq, sx, *ex["gate"], off)
+    u = O.grouped_gemm(xq, sx, *ex["up"], off)
+    rhq, rsh = O.quant_act_group((O.silu(g) * u).astype(np.float32))
+    assert np.allclose(sh.cpu().numpy(), rsh, rtol=1e-3)
+    assert np.mean(H.codes_np(hq) != rhq) < 5e-3
+    y = jg.gemm_down(H.to_cuda(rhq), H.to_cuda(rsh), dex["down_proj"], H.to_cuda(off))
+    want_y = O.bf16_round(O.grouped_gemm(rhq, rsh, *ex["down"], off).astype(np.float32))
+    H.assert_close_out(H.bf16_to_np(y), want_y, tol=1e-2)
