@@ -27,15 +27,31 @@ __device__ __forceinline__ unsigned key_index(unsigned long long key) {
   return 0xffffffffu - (unsigned)(key & 0xffffffffu);
 }
 
+// Wave-wide maximum of 64-bit keys, result in every lane.  Inside a row of 16 lanes the partners are reached with
+// DPP lane permutations (a few cycles each: xor 1, xor 2, mirror of 8, mirror of 16 -- a maximum does not care
+// which partner it meets, only that the set closes); the four row maxima are then read as scalars.  The same
+// reduction over ds_bpermute takes about 100 cycles per step, and routing is a chain of some thirty reductions.
+template <int CTRL> __device__ __forceinline__ unsigned long long dpp_max_u64(unsigned long long k) {
+  const int lo = (int)(unsigned)(k & 0xffffffffu), hi = (int)(unsigned)(k >> 32);
+  const unsigned olo = (unsigned)__builtin_amdgcn_update_dpp(lo, lo, CTRL, 0xF, 0xF, false);
+  const unsigned ohi = (unsigned)__builtin_amdgcn_update_dpp(hi, hi, CTRL, 0xF, 0xF, false);
+  const unsigned long long o = ((unsigned long long)ohi << 32) | olo;
+  return o > k ? o : k;
+}
 __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long k) {
+  k = dpp_max_u64<0xB1>(k);    // quad_perm [1,0,3,2]: lane ^ 1
+  k = dpp_max_u64<0x4E>(k);    // quad_perm [2,3,0,1]: lane ^ 2
+  k = dpp_max_u64<0x141>(k);   // row_half_mirror: lane i <-> 7 - i within 8
+  k = dpp_max_u64<0x140>(k);   // row_mirror: lane i <-> 15 - i within 16
+  unsigned long long best = 0ull;
 #pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) {
-    unsigned lo = __shfl_xor((unsigned)(k & 0xffffffffu), off, MOE_WAVE);
-    unsigned hi = __shfl_xor((unsigned)(k >> 32), off, MOE_WAVE);
-    unsigned long long o = ((unsigned long long)hi << 32) | lo;
-    k = o > k ? o : k;
+  for (int r = 0; r < 4; ++r) {
+    const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(k & 0xffffffffu), 16 * r);
+    const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(k >> 32), 16 * r);
+    const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+    best = o > best ? o : best;
   }
-  return k;
+  return best;
 }
 __device__ __forceinline__ float wave_max_f32(float v) {
 #pragma unroll
