@@ -58,7 +58,7 @@ def make_weights(jg, torch, E, N, K, gen, std=0.02, chunk=16):
     return {"w": wq, "scale_inv": sw}
 
 
-def make_layer(jg, torch, cfg, seed=0):
+def make_layer(jg, torch, cfg, seed=0, bias_std=0.1):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
     D, E, I, SI = cfg["D"], cfg["E"], cfg["I"], cfg["SI"]
@@ -70,7 +70,7 @@ def make_layer(jg, torch, cfg, seed=0):
                       down_proj=make_weights(jg, torch, 1, D, SI, gen))
     bias = None
     if cfg["routing"] == "sigmoid_grouped":
-        bias = torch.randn((E,), dtype=torch.float32, device="cuda", generator=gen) * 0.1
+        bias = torch.randn((E,), dtype=torch.float32, device="cuda", generator=gen) * bias_std
     return experts, shared, bias, gen
 
 
@@ -186,6 +186,9 @@ def main():
     ap.add_argument("--workload", default="deepseek_v3_prefill", choices=sorted(WORKLOADS))
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--bias-std", type=float, default=0.1,
+                    help="standard deviation of the selection bias of sigmoid_grouped routing (0.1 = the workload as "
+                         "specified: the same 7 of 8 groups win almost every token; 0 = balanced routing)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (expert parallelism is shown as one "
@@ -204,7 +207,7 @@ def main():
 
     cfg = WORKLOADS[args.workload]
     t0 = time.perf_counter()
-    layer = make_layer(jg, torch, cfg)
+    layer = make_layer(jg, torch, cfg, bias_std=args.bias_std)
     torch.cuda.synchronize()
     log(f"weights for {args.workload} generated in {time.perf_counter() - t0:.1f} s")
     main_res = run_workload(jg, torch, args.workload, cfg, layer, args.steps, args.warmup)
@@ -235,7 +238,7 @@ def main():
         "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp8_e4m3", "data": "synthetic",
         "config": {"workload": args.workload, **{k: cfg[k] for k in ("M", "D", "E", "k", "I", "SI", "routing")},
-                   "touched_experts": main_res["touched_experts"]},
+                   "touched_experts": main_res["touched_experts"], "bias_std": args.bias_std},
         "frac_of_peak": (value / PEAK_HBM_GBS) if is_decode else (value / PEAK_FP8_TFLOPS),
         "graph_replay_ms_per_step": main_res["graph_ms_per_step"],
         "roofline": roof,
