@@ -579,3 +579,46 @@ def test_grouped_gemms_random_group_sizes(jg, seed):
     y = jg.gemm_down(H.to_cuda(rhq), H.to_cuda(rsh), dex["down_proj"], H.to_cuda(off))
     want_y = O.bf16_round(O.grouped_gemm(rhq, rsh, *ex["down"], off).astype(np.float32))
     H.assert_close_out(H.bf16_to_np(y), want_y, tol=1e-2)
+
+
+def test_concurrent_calls_on_two_streams(jg):
+    """Two host threads, each with its own stream and workspace, call the layer at the same time (the library's
+    only shared state is the per-device side stream and the thread-local error text): every result equals the one
+    the same inputs give when the calls run one after the other."""
+    import threading
+    import torch
+    _say("concurrent streams")
+    probs = [H.make_problem(M=300, D=512, E=16, k=4, I=256, SI=128, seed=60),
+             H.make_problem(M=64, D=1024, E=32, k=2, I=384, SI=256, seed=61)]
+    cases = []
+    for prob, k in zip(probs, (4, 2)):
+        ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
+        x = H.to_bf16_cuda(prob["x"]); lg = H.to_cuda(prob["logits"])
+        serial = jg.moe_experts(x, lg, top_k=k, experts=ex, shared=sh)
+        cases.append((x, lg, k, ex, sh, serial))
+    torch.cuda.synchronize()
+    results = [[], []]
+    errors = []
+
+    def worker(i):
+        try:
+            x, lg, k, ex, sh, _ = cases[i]
+            s = torch.cuda.Stream()
+            with torch.cuda.stream(s):
+                for _ in range(20):
+                    results[i].append(jg.moe_experts(x, lg, top_k=k, experts=ex, shared=sh))
+            s.synchronize()
+        except Exception as exc:   # surfaced below: an exception in a thread would otherwise pass silently
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for i in range(2):
+        assert len(results[i]) == 20
+        for out in results[i]:
+            assert torch.equal(out, cases[i][5])
