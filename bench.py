@@ -229,7 +229,7 @@ def main():
     else:
         metric, value, unit = "MoE layer fp8 TFLOP/s (prefill)", main_res["tflops"], "TFLOP/s"
         roof = {"bound": "mfma", "achieved": gk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC.get(args.workload),
+                "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC.get(args.workload) if args.bias_std == 0.1 else None,
                 "kernel": "grouped_gemm_kernel<0, 2>, routed launch (gate/up + SwiGLU + h quantisation)",
                 "algorithmic_bytes_per_launch": gk["bytes_per_launch"],
                 "avg_launch_ms": gk["avg_launch_ms"], "flops_per_launch": gk["flops_per_launch"]}
