@@ -145,7 +145,7 @@ typedef struct MoeForwardArgs {
   const void* w_router;          /* (E, D) bf16: logits = bf16(x . w_router^T), moe.py:50 */
   const void* w_shared_gate;     /* (1, D) bf16 or NULL: shared expert's output is scaled by
                                     sigmoid(x . w_shared_gate^T), moe.py:278-279; needs w_router and SI > 0 */
-  float* out_logits;             /* (M, E) optional debug output of the computed logits */
+  float* out_logits;             /* (M, E) optional copy of the logits the router computed (else never stored) */
   /* the steps either side of the layer (block.py:54-58, :88-91); NULL / 0 = off */
   const float* norm_weight;      /* (D) f32: x is RMS-normalised first (rms_norm with 1 + weight, in bf16) */
   float norm_eps;

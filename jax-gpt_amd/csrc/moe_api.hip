@@ -65,7 +65,7 @@ struct Carver {
 
 struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
-  float *w, *sx, *sh, *shs, *logits, *shared_gate;
+  float *w, *sx, *sh, *shs, *shared_gate;
   uint8_t *xq, *hq, *hsq;
   void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared, *router_ws, *normed;
   size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, router_ws_bytes, total;
@@ -98,7 +98,6 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool r
   b.hsq = SI ? (uint8_t*)c.take((size_t)M * SI) : nullptr;
   b.shs = SI ? (float*)c.take((size_t)M * (SI / 128) * 4) : nullptr;
   b.ys = SI ? c.take((size_t)M * D * 2) : nullptr;
-  b.logits = router ? (float*)c.take((size_t)M * E * 4) : nullptr;
   b.shared_gate = router ? (float*)c.take((size_t)M * 4) : nullptr;
   b.router_ws_bytes = router ? moe_router_workspace_bytes(M, D, E) : 0;
   b.router_ws = router ? c.take(b.router_ws_bytes) : nullptr;
@@ -201,27 +200,29 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     return moe_check_hip(e2, "forward: join");
   };
 
-  const float* logits = a->logits;
+  // With a router weight the routing kernel adds the matmul's split-K partial sums itself: the (M, E) logits
+  // are written only when out_logits asks for them.
+  LogitSource src{a->logits, nullptr, 0, a->E, nullptr, nullptr};
   const float* shared_gate = nullptr;
   if (a->w_router) {
-    float* lg = a->out_logits ? a->out_logits : b.logits;
     // the router reads the normalised activations, which the (possibly forked) quantiser writes
     if (a->norm_weight && !quant_joined) {
       if (rc_shared) return join(rc_shared);
       if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
       quant_joined = true;
     }
-    if ((rc = moe_router_logits(a->norm_weight ? b.normed : a->x, a->M, a->D, a->w_router, a->E, a->w_shared_gate, lg,
-                                a->w_shared_gate ? b.shared_gate : nullptr, b.router_ws, b.router_ws_bytes, stream)))
+    int splits = 0, n_cols = 0;
+    if ((rc = moe_router_partials(a->norm_weight ? b.normed : a->x, a->M, a->D, a->w_router, a->E, a->w_shared_gate,
+                                  b.router_ws, b.router_ws_bytes, &splits, &n_cols, stream)))
       return join(rc);
-    logits = lg;
     if (a->w_shared_gate) shared_gate = b.shared_gate;
+    src = LogitSource{nullptr, (const float*)b.router_ws, splits, n_cols, a->out_logits, b.shared_gate};
   }
   if (a->routing == MOE_ROUTING_SOFTMAX)
-    rc = moe_route_softmax_topk(logits, a->M, a->E, a->k, a->renorm, idx, w, stream);
+    rc = moe_route_softmax_impl(src, a->M, a->E, a->k, a->renorm, idx, w, stream);
   else
-    rc = moe_route_sigmoid_grouped(logits, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
-                                   a->routed_scale, idx, w, stream);
+    rc = moe_route_sigmoid_grouped_impl(src, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
+                                        a->routed_scale, idx, w, stream);
   if (rc) return join(rc);
   if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
                         b.permute_ws_bytes, stream)))

@@ -67,6 +67,24 @@ __device__ inline void moe_write_expert_items(const ListSpec& spec, int expert, 
 }
 
 // grouped GEMMs with an optional pre-built work list (moe_gemm.hip); the extern "C" entry points build their own
+// Where the routing kernels take a token's logits from: an (M, E) array, or the router matmul's split-K partial
+// sums [splits][M][N] (N = E, + 1 when the shared expert's gate is the last column), which they add in slice order
+// and round to bf16 themselves -- the logits then never travel through memory unless out_logits asks for them.
+struct LogitSource {
+  const float* logits;    // (M, E), used when partial is null
+  const float* partial;   // [splits][M][N] or null
+  int splits, N;
+  float* out_logits;      // optional (M, E) copy of what the kernel ranked (partial mode only)
+  float* shared_gate;     // (M) sigmoid of column E, written in partial mode when N > E
+};
+int moe_router_partials(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
+                        const void* w_shared_gate_bf16, void* ws, size_t ws_bytes, int* splits_used, int* n_cols,
+                        moe_stream_t stream);
+int moe_route_softmax_impl(const LogitSource& src, int M, int E, int k, int renorm, int32_t* idx, float* w,
+                           moe_stream_t stream);
+int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, int M, int E, int n_group,
+                                   int topk_group, int k, int renorm, float routed_scale, int32_t* idx, float* w,
+                                   moe_stream_t stream);
 int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
                          size_t ws_bytes_each, moe_stream_t stream);
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,

@@ -66,15 +66,35 @@ __device__ __forceinline__ float wave_sum_f32(float v) {
 
 constexpr int kWavesPerBlock = 4;
 
+// Logit (t, e).  In partial mode: the slices added in slice order, one bf16 rounding (what the router's own
+// finishing pass computes, moe_router.hip), optionally copied out.
+__device__ __forceinline__ float fetch_logit(const LogitSource& src, int M, int E, int t, int e) {
+  if (!src.partial) return src.logits[(size_t)t * E + e];
+  const size_t MN = (size_t)M * src.N, at = (size_t)t * src.N + e;
+  float s = src.partial[at];
+  for (int z = 1; z < src.splits; ++z) s = __fadd_rn(s, src.partial[(size_t)z * MN + at]);
+  const float v = bf16_to_f32(f32_to_bf16(s));
+  if (src.out_logits) src.out_logits[(size_t)t * E + e] = v;
+  return v;
+}
+// the shared expert's gate rides in column E of the partial sums: one lane per token finishes it
+__device__ __forceinline__ void finish_shared_gate(const LogitSource& src, int M, int E, int t) {
+  if (!src.partial || !src.shared_gate || src.N <= E) return;
+  const size_t MN = (size_t)M * src.N, at = (size_t)t * src.N + E;
+  float s = src.partial[at];
+  for (int z = 1; z < src.splits; ++z) s = __fadd_rn(s, src.partial[(size_t)z * MN + at]);
+  src.shared_gate[t] = bf16_to_f32(f32_to_bf16(sigmoid_det(bf16_to_f32(f32_to_bf16(s)))));
+}
+
 // VPL = values per lane; element e lives in lane e%64, slot e/64.
 template <int VPL>
 __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_softmax_kernel(
-    const float* __restrict__ logits, int M, int E, int k, int renorm, int32_t* __restrict__ idx,
+    const LogitSource src, int M, int E, int k, int renorm, int32_t* __restrict__ idx,
     float* __restrict__ w) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (t >= M) return;
-  const float* row = logits + (size_t)t * E;
+  if (lane == 0) finish_shared_gate(src, M, E, t);
   float v[VPL];
   unsigned long long key[VPL];
   float mx = -INFINITY;
@@ -82,7 +102,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_softmax_kernel
   for (int s = 0; s < VPL; ++s) {
     int e = lane + 64 * s;
     bool ok = e < E;
-    v[s] = ok ? row[e] : -INFINITY;
+    v[s] = ok ? fetch_logit(src, M, E, t, e) : -INFINITY;
     key[s] = ok ? make_key(v[s], (unsigned)e) : 0ull;
     mx = fmaxf(mx, v[s]);
   }
@@ -119,13 +139,13 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_softmax_kernel
 
 template <int VPL>
 __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_grouped_kernel(
-    const float* __restrict__ logits, const float* __restrict__ bias, int M, int E, int n_group,
+    const LogitSource src, const float* __restrict__ bias, int M, int E, int n_group,
     int topk_group, int k, int renorm, float routed_scale, int32_t* __restrict__ idx,
     float* __restrict__ w) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (t >= M) return;
-  const float* row = logits + (size_t)t * E;
+  if (lane == 0) finish_shared_gate(src, M, E, t);
   const int per = E / n_group;
   float score[VPL];
   unsigned long long key[VPL];
@@ -134,7 +154,7 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
   for (int s = 0; s < VPL; ++s) {
     int e = lane + 64 * s;
     bool ok = e < E;
-    score[s] = ok ? sigmoid_det(row[e]) : 0.f;
+    score[s] = ok ? sigmoid_det(fetch_logit(src, M, E, t, e)) : 0.f;
     float choice = __fadd_rn(score[s], (ok && bias) ? bias[e] : 0.f);
     key[s] = ok ? make_key(choice, (unsigned)e) : 0ull;
     gid[s] = ok ? e / per : -1;
@@ -201,8 +221,9 @@ __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_groupe
   }
 }
 
-int check_route_args(const float* logits, int M, int E, int k, const int32_t* idx, const float* w) {
-  MOE_REQUIRE(M == 0 || (logits && idx && w), MOE_ERR_NULL, "route: null pointer");
+int check_route_args(const LogitSource& src, int M, int E, int k, const int32_t* idx, const float* w) {
+  MOE_REQUIRE(M == 0 || ((src.logits || src.partial) && idx && w), MOE_ERR_NULL, "route: null pointer");
+  MOE_REQUIRE(!src.partial || (src.splits >= 1 && src.N >= E), MOE_ERR_BAD_SHAPE, "route: bad partial-sum layout");
   MOE_REQUIRE(M >= 0 && E >= 1 && E <= 1024, MOE_ERR_BAD_SHAPE, "route: need 1 <= E <= 1024, got E=%d M=%d", E, M);
   MOE_REQUIRE(k >= 1 && k <= 32 && k <= E, MOE_ERR_BAD_SHAPE, "route: need 1 <= k <= min(32,E), got k=%d E=%d", k, E);
   return MOE_OK;
@@ -221,21 +242,25 @@ int check_route_args(const float* logits, int M, int E, int k, const int32_t* id
     else hipLaunchKernelGGL(KERNEL<16>, grid, block, 0, s, __VA_ARGS__);                  \
   } while (0)
 
-extern "C" int moe_route_softmax_topk(const float* logits, int M, int E, int k, int renorm,
-                                      int32_t* idx, float* w, moe_stream_t stream) {
-  int rc = check_route_args(logits, M, E, k, idx, w);
+int moe_route_softmax_impl(const LogitSource& src, int M, int E, int k, int renorm, int32_t* idx, float* w,
+                           moe_stream_t stream) {
+  int rc = check_route_args(src, M, E, k, idx, w);
   if (rc) return rc;
   if (M == 0) return MOE_OK;
   hipStream_t s = (hipStream_t)stream;
-  DISPATCH_VPL(E, route_softmax_kernel, logits, M, E, k, renorm, idx, w);
+  DISPATCH_VPL(E, route_softmax_kernel, src, M, E, k, renorm, idx, w);
   return moe_check_hip(hipGetLastError(), "route_softmax launch");
 }
 
-extern "C" int moe_route_sigmoid_grouped(const float* logits, const float* bias, int M, int E,
-                                         int n_group, int topk_group, int k, int renorm,
-                                         float routed_scale, int32_t* idx, float* w,
-                                         moe_stream_t stream) {
-  int rc = check_route_args(logits, M, E, k, idx, w);
+extern "C" int moe_route_softmax_topk(const float* logits, int M, int E, int k, int renorm,
+                                      int32_t* idx, float* w, moe_stream_t stream) {
+  return moe_route_softmax_impl(LogitSource{logits, nullptr, 0, E, nullptr, nullptr}, M, E, k, renorm, idx, w, stream);
+}
+
+int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, int M, int E, int n_group,
+                                   int topk_group, int k, int renorm, float routed_scale, int32_t* idx, float* w,
+                                   moe_stream_t stream) {
+  int rc = check_route_args(src, M, E, k, idx, w);
   if (rc) return rc;
   MOE_REQUIRE(n_group >= 1 && n_group <= 64 && E % n_group == 0, MOE_ERR_BAD_SHAPE,
               "route: n_group=%d must divide E=%d and be <= 64", n_group, E);
@@ -245,7 +270,15 @@ extern "C" int moe_route_sigmoid_grouped(const float* logits, const float* bias,
               "route: k=%d exceeds the %d experts of the kept groups", k, topk_group * (E / n_group));
   if (M == 0) return MOE_OK;
   hipStream_t s = (hipStream_t)stream;
-  DISPATCH_VPL(E, route_sigmoid_grouped_kernel, logits, bias, M, E, n_group, topk_group, k, renorm,
+  DISPATCH_VPL(E, route_sigmoid_grouped_kernel, src, bias, M, E, n_group, topk_group, k, renorm,
                routed_scale, idx, w);
   return moe_check_hip(hipGetLastError(), "route_sigmoid_grouped launch");
+}
+
+extern "C" int moe_route_sigmoid_grouped(const float* logits, const float* bias, int M, int E,
+                                         int n_group, int topk_group, int k, int renorm,
+                                         float routed_scale, int32_t* idx, float* w,
+                                         moe_stream_t stream) {
+  return moe_route_sigmoid_grouped_impl(LogitSource{logits, nullptr, 0, E, nullptr, nullptr}, bias, M, E, n_group,
+                                        topk_group, k, renorm, routed_scale, idx, w, stream);
 }

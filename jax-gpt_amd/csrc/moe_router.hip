@@ -146,12 +146,11 @@ extern "C" size_t moe_router_workspace_bytes(int M, int D, int E) {
   return (size_t)choose_splits(M, N, D) * (size_t)M * N * sizeof(float) + 256;
 }
 
-extern "C" int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
-                                 const void* w_shared_gate_bf16, float* logits, float* shared_gate, void* ws,
-                                 size_t ws_bytes, moe_stream_t stream) {
-  MOE_REQUIRE((M == 0 || (x_bf16 && logits)) && w_router_bf16 && ws, MOE_ERR_NULL, "router: null pointer");
-  MOE_REQUIRE((w_shared_gate_bf16 == nullptr) == (shared_gate == nullptr), MOE_ERR_NULL,
-              "router: the shared gate's weight and output come together");
+// The matmul alone: split-K partial sums [splits][M][N] at the start of ws (N = E, + 1 with the gate column).
+int moe_router_partials(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
+                        const void* w_shared_gate_bf16, void* ws, size_t ws_bytes, int* splits_used, int* n_cols,
+                        moe_stream_t stream) {
+  MOE_REQUIRE((M == 0 || x_bf16) && w_router_bf16 && ws, MOE_ERR_NULL, "router: null pointer");
   MOE_REQUIRE(M >= 0 && D > 0 && D % 128 == 0 && E >= 1 && E <= 1024, MOE_ERR_BAD_SHAPE,
               "router: need D %% 128 == 0 and 1 <= E <= 1024, got M=%d D=%d E=%d", M, D, E);
   MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(w_router_bf16) && MOE_ALIGNED16(w_shared_gate_bf16) &&
@@ -159,13 +158,14 @@ extern "C" int moe_router_logits(const void* x_bf16, int M, int D, const void* w
               MOE_ERR_BAD_ALIGN, "router: pointers must be 16-byte aligned");
   MOE_REQUIRE(ws_bytes >= moe_router_workspace_bytes(M, D, E), MOE_ERR_WORKSPACE_TOO_SMALL,
               "router: workspace %zu < %zu", ws_bytes, moe_router_workspace_bytes(M, D, E));
-  if (M == 0) return MOE_OK;
   const int N = E + (w_shared_gate_bf16 ? 1 : 0);
   const int splits = choose_splits(M, N, D);
   const int k_per_split = ((D / RBK + splits - 1) / splits) * RBK;
   const int used = (D + k_per_split - 1) / k_per_split;   // slices that hold at least one K step
+  *splits_used = used;
+  *n_cols = N;
+  if (M == 0) return MOE_OK;
   MOE_REQUIRE((long long)M * D * 2 < (1ll << 32), MOE_ERR_BAD_SHAPE, "router: the activations must stay within 4 GB");
-  float* partial = (float*)ws;
   hipStream_t s = (hipStream_t)stream;
   static bool attr_set = false;
   if (!attr_set) {
@@ -175,9 +175,21 @@ extern "C" int moe_router_logits(const void* x_bf16, int M, int D, const void* w
   }
   hipLaunchKernelGGL(router_gemm_kernel, dim3((M + RT - 1) / RT, (N + RN - 1) / RN, used), dim3(256), R_LDS, s,
                      (const bf16_t*)x_bf16, M, D, (const bf16_t*)w_router_bf16, E, (const bf16_t*)w_shared_gate_bf16, N,
-                     k_per_split, partial);
+                     k_per_split, (float*)ws);
+  return moe_check_hip(hipGetLastError(), "router launch");
+}
+
+extern "C" int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
+                                 const void* w_shared_gate_bf16, float* logits, float* shared_gate, void* ws,
+                                 size_t ws_bytes, moe_stream_t stream) {
+  MOE_REQUIRE(M == 0 || logits, MOE_ERR_NULL, "router: null pointer");
+  MOE_REQUIRE((w_shared_gate_bf16 == nullptr) == (shared_gate == nullptr), MOE_ERR_NULL,
+              "router: the shared gate's weight and output come together");
+  int used = 0, N = 0;
+  int rc = moe_router_partials(x_bf16, M, D, w_router_bf16, E, w_shared_gate_bf16, ws, ws_bytes, &used, &N, stream);
+  if (rc || M == 0) return rc;
   const long long total = (long long)M * N;
-  hipLaunchKernelGGL(router_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, partial, M, E, N,
-                     used, logits, shared_gate);
+  hipLaunchKernelGGL(router_finish_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const float*)ws, M, E, N, used, logits, shared_gate);
   return moe_check_hip(hipGetLastError(), "router launch");
 }
