@@ -1,6 +1,8 @@
 // Shared device/host helpers for the gfx950 MoE kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include "moe_hip.h"
@@ -17,6 +19,20 @@ typedef unsigned short bf16_t;  // raw bf16 bits
 // host side: record an error message for moe_last_error() and return the code
 int moe_set_error(int code, const char* fmt, ...);
 int moe_check_hip(hipError_t e, const char* what);
+
+// hipFuncSetAttribute applies to the current device: remember, per kernel, on which devices the dynamic LDS limit
+// has been raised (bit d of the mask = device d; safe to call from several host threads).
+inline int moe_raise_lds_limit(const void* kernel, int bytes, std::atomic<unsigned long long>& done_mask) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return moe_check_hip(e, "hipGetDevice");
+  const unsigned long long bit = 1ull << (dev & 63);
+  if (done_mask.load(std::memory_order_acquire) & bit) return MOE_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return moe_check_hip(e, "raising the dynamic LDS limit");
+  done_mask.fetch_or(bit, std::memory_order_release);
+  return MOE_OK;
+}
 
 // ---- work list of the grouped GEMMs ----
 struct WorkHeader {

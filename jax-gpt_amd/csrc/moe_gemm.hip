@@ -495,13 +495,8 @@ int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const
     const ListSpec spec{ncb, max_items, hdr, items};
     hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, C::BM, spec, spec);
   }
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t err = hipFuncSetAttribute((const void*)grouped_gemm_kernel<MODE, XW>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-    if (err != hipSuccess) return moe_check_hip(err, "gemm: raising the dynamic LDS limit");
-    attr_set = true;
-  }
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE, XW>, C::LDS_BYTES, lds_raised)) return rc;
   const int grid = ((max_items + 7) / 8) * 8;
   hipLaunchKernelGGL((grouped_gemm_kernel<MODE, XW>), dim3(grid), dim3(NT), C::LDS_BYTES, s, xq, sx, row_ids, w0, sw0,
                      w1, sw1, hdr, items, K, N, out, out_scale);

@@ -167,12 +167,8 @@ int moe_router_partials(const void* x_bf16, int M, int D, const void* w_router_b
   if (M == 0) return MOE_OK;
   MOE_REQUIRE((long long)M * D * 2 < (1ll << 32), MOE_ERR_BAD_SHAPE, "router: the activations must stay within 4 GB");
   hipStream_t s = (hipStream_t)stream;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t err = hipFuncSetAttribute((const void*)router_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, R_LDS);
-    if (err != hipSuccess) return moe_check_hip(err, "router: raising the dynamic LDS limit");
-    attr_set = true;
-  }
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (int rc = moe_raise_lds_limit((const void*)router_gemm_kernel, R_LDS, lds_raised)) return rc;
   hipLaunchKernelGGL(router_gemm_kernel, dim3((M + RT - 1) / RT, (N + RN - 1) / RN, used), dim3(256), R_LDS, s,
                      (const bf16_t*)x_bf16, M, D, (const bf16_t*)w_router_bf16, E, (const bf16_t*)w_shared_gate_bf16, N,
                      k_per_split, (float*)ws);
