@@ -67,7 +67,7 @@ struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
   float *w, *sx, *sh, *shs, *shared_gate;
   uint8_t *xq, *hq, *hsq;
-  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_down, *gemm_ws_shared, *router_ws, *normed;
+  void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_shared, *router_ws, *normed;
   size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, router_ws_bytes, total;
 };
 
@@ -85,8 +85,7 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool r
   b.permute_ws_bytes = moe_permute_workspace_bytes(M, k, E);
   b.permute_ws = c.take(b.permute_ws_bytes);
   b.gemm_ws_bytes = moe_gemm_workspace_bytes((int)R, E, I > D ? I : D);
-  b.gemm_ws = c.take(b.gemm_ws_bytes);        // work list of the routed gate/up GEMM
-  b.gemm_ws_down = c.take(b.gemm_ws_bytes);   // ... of the routed down GEMM (both are listed in one launch)
+  b.gemm_ws = c.take(b.gemm_ws_bytes);        // tile list of the routed GEMMs (gate/up and down share it)
   // the shared expert runs beside the routed ones on its own stream: its launches need their own work lists
   b.gemm_ws_shared_bytes = SI ? moe_gemm_workspace_bytes(M, 1, SI > D ? SI : D) : 0;
   b.gemm_ws_shared = SI ? c.take(b.gemm_ws_shared_bytes) : nullptr;
@@ -178,12 +177,12 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
     if (!rc_shared)
-      rc_shared = moe_gemm_gateup_swiglu_fp8(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up,
-                                             b.dense_off, 1, a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws_shared,
-                                             b.gemm_ws_shared_bytes, (moe_stream_t)side);
-    if (!rc_shared)
-      rc_shared = moe_gemm_down_fp8(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
-                                    b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
+      rc_shared = moe_gemm_gateup_impl(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up, b.dense_off, 1,
+                                       a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, false,
+                                       (moe_stream_t)side);
+    if (!rc_shared)   // same rows, same tile height: the list the gate/up launch built serves the down launch too
+      rc_shared = moe_gemm_down_impl(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
+                                     b.gemm_ws_shared, b.gemm_ws_shared_bytes, true, (moe_stream_t)side);
   } else {
     if ((rc = quantise(a, b, stream))) return rc;
   }
@@ -227,9 +226,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
                         b.permute_ws_bytes, stream)))
     return join(rc);
-  if ((rc = moe_gemm_build_lists(b.group_offsets, a->E, R, a->D, a->I, b.gemm_ws, b.gemm_ws_down, b.gemm_ws_bytes,
-                                 stream)))
-    return join(rc);
+  if ((rc = moe_gemm_build_tiles(b.group_offsets, a->E, R, b.gemm_ws, b.gemm_ws_bytes, stream))) return join(rc);
   if (!quant_joined) {
     if (rc_shared) return join(rc_shared);
     if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
@@ -238,7 +235,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
                                  a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = moe_gemm_down_impl(b.hq, b.sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
-                               b.gemm_ws_down, b.gemm_ws_bytes, true, stream)))
+                               b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;
   return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, shared_gate, a->add_residual ? a->x : nullptr, a->M, a->k,

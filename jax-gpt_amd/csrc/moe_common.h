@@ -35,17 +35,20 @@ inline int moe_raise_lds_limit(const void* kernel, int bytes, std::atomic<unsign
 }
 
 // ---- work list of the grouped GEMMs ----
-struct WorkHeader {
-  int n_items;
+// One entry per row tile, in [expert][tile] order; every entry carries its EXPERT's row range and the index of the
+// expert's first tile, from which a workgroup derives its own tile and column block (moe_gemm.hip).  The list
+// depends on the group sizes and the tile height only, so the gate/up and the down GEMM of a layer share it.
+struct TileHeader {
+  int n_tiles;
   int pad[3];
 };
-struct WorkItem {
-  int expert, row_start, row_count, col_block;
+struct TileEntry {
+  int expert, row_start, rows, first_tile;
 };
-struct ListSpec {
-  int n_col_blocks, max_items;   // n_col_blocks == 0: no list wanted
-  WorkHeader* hdr;
-  WorkItem* items;
+struct TileList {
+  int max_tiles;
+  TileHeader* hdr;
+  TileEntry* tiles;
 };
 // An expert with `rows` rows gets ceil(rows / bm) row tiles of equal height (a multiple of 16, the last one
 // shorter): tiles that share a weight slab then take the same time per K step and walk it together, so the
@@ -62,27 +65,6 @@ __host__ __device__ inline int moe_tile_count(int rows, int bm) {
   const int tr = moe_tile_rows(rows, bm);
   return (rows + tr - 1) / tr;
 }
-// the items of one expert, [col_block][row tile] from position tile_base * n_col_blocks on; `first` / `step` let a
-// group of threads share the expert
-__device__ inline void moe_write_expert_items(const ListSpec& spec, int expert, int row_start, int rows, int tile_base,
-                                              int bm, int first, int step) {
-  const int tiles = moe_tile_count(rows, bm);
-  const int tr = moe_tile_rows(rows, bm);
-  const int n = tiles * spec.n_col_blocks;
-  for (int local = first; local < n; local += step) {
-    const int it = tile_base * spec.n_col_blocks + local;
-    if (it >= spec.max_items) break;   // cannot happen for consistent offsets; keeps writes in bounds
-    const int cb = tiles == 1 ? local : local / tiles, rt = tiles == 1 ? 0 : local - cb * tiles;
-    WorkItem w;
-    w.expert = expert;
-    w.row_start = row_start + rt * tr;
-    w.row_count = min(tr, rows - rt * tr);
-    w.col_block = cb;
-    spec.items[it] = w;
-  }
-}
-
-// grouped GEMMs with an optional pre-built work list (moe_gemm.hip); the extern "C" entry points build their own
 // Where the routing kernels take a token's logits from: an (M, E) array, or the router matmul's split-K partial
 // sums [splits][M][N] (N = E, + 1 when the shared expert's gate is the last column), which they add in slice order
 // and round to bf16 themselves -- the logits then never travel through memory unless out_logits asks for them.
@@ -101,8 +83,8 @@ int moe_route_softmax_impl(const LogitSource& src, int M, int E, int k, int reno
 int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, int M, int E, int n_group,
                                    int topk_group, int k, int renorm, float routed_scale, int32_t* idx, float* w,
                                    moe_stream_t stream);
-int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
-                         size_t ws_bytes_each, moe_stream_t stream);
+// grouped GEMMs with an optional pre-built tile list in ws (moe_gemm.hip); the extern "C" entry points build their own
+int moe_gemm_build_tiles(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream);
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
                          const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
                          int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,

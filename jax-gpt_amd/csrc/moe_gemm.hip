@@ -35,12 +35,13 @@
 // The copies of a step are issued a few at a time between MFMA groups, not in
 // one burst, and the two waves of each SIMD run out of phase (see the K loop).
 //
-// Work items are listed on the device by build_items_kernel (no host read-back
-// of group sizes) in [expert][column block][row tile] order and dealt to the 8
-// XCDs in contiguous ranges, so the row tiles and column blocks that share a
-// weight slab or an activation tile run together under one L2.  An expert's
-// rows are cut into tiles of equal height, so that the tiles sharing a weight
-// slab advance at the same pace.
+// Row tiles are listed on the device by build_tiles_kernel (no host read-back
+// of group sizes); a workgroup's work item is a (row tile, column block) pair
+// derived from its index, in [expert][column block][row tile] order, and the
+// items are dealt to the 8 XCDs in contiguous ranges, so the row tiles and
+// column blocks that share a weight slab or an activation tile run together
+// under one L2.  An expert's rows are cut into tiles of equal height, so that
+// the tiles sharing a weight slab advance at the same pace.
 #include <stdlib.h>
 
 #include <type_traits>
@@ -58,18 +59,17 @@ constexpr int MODE_DOWN = 1;
 
 // ---- work list -----------------------------------------------------------
 
-// Workgroup b builds list b (the gate/up and the down GEMM of one layer walk the same rows with different
-// column-block counts: one launch lists both).  Item order [expert][col_block][row tile]; each wave writes the
-// items of the experts it owns.
-__global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __restrict__ group_offsets, int E, int bm,
-                                                          ListSpec l0, ListSpec l1) {
-  const ListSpec spec = blockIdx.x == 0 ? l0 : l1;
-  __shared__ int tile_prefix[1025];
+// One workgroup lists the row tiles of every expert, [expert][tile]; thread e owns expert e.
+__global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __restrict__ group_offsets, int E, int bm,
+                                                          TileList l) {
   __shared__ int wave_tot[16];
   const int e = threadIdx.x;
   const int lane = e & 63, wv = e >> 6;
-  int rows = 0;
-  if (e < E) rows = group_offsets[e + 1] - group_offsets[e];
+  int start = 0, rows = 0;
+  if (e < E) {
+    start = group_offsets[e];
+    rows = group_offsets[e + 1] - start;
+  }
   const int tiles = moe_tile_count(rows, bm);
   int incl = tiles;
 #pragma unroll
@@ -79,18 +79,15 @@ __global__ __launch_bounds__(1024) void build_items_kernel(const int32_t* __rest
   }
   if (lane == 63) wave_tot[wv] = incl;
   __syncthreads();
-  int wbase = 0;
-  for (int i = 0; i < wv; ++i) wbase += wave_tot[i];
-  if (e < E) tile_prefix[e + 1] = wbase + incl;
-  if (e == 0) tile_prefix[0] = 0;
-  __syncthreads();
-  int total = tile_prefix[E] * spec.n_col_blocks;
-  if (total > spec.max_items) total = spec.max_items;
-  if (e == 0) spec.hdr->n_items = total;
-  for (int x = wv; x < E; x += 16) {
-    const int start = group_offsets[x], rows_x = group_offsets[x + 1] - start;
-    if (rows_x > 0) moe_write_expert_items(spec, x, start, rows_x, tile_prefix[x], bm, lane, MOE_WAVE);
+  int wbase = 0, total = 0;
+  for (int i = 0; i < 16; ++i) {
+    if (i < wv) wbase += wave_tot[i];
+    total += wave_tot[i];
   }
+  const int first = wbase + incl - tiles;
+  for (int t = 0; t < tiles; ++t)
+    if (first + t < l.max_tiles) l.tiles[first + t] = TileEntry{e, start, rows, first};   // (cannot overflow for consistent offsets)
+  if (e == 0) l.hdr->n_tiles = total < l.max_tiles ? total : l.max_tiles;
 }
 
 // ---- main kernel ---------------------------------------------------------
@@ -171,7 +168,7 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0,   // gate (GATEUP) or down (DOWN)
     const uint8_t* __restrict__ w1, const float* __restrict__ sw1,   // up (GATEUP only)
-    const WorkHeader* __restrict__ hdr, const WorkItem* __restrict__ items,
+    const TileHeader* __restrict__ hdr, const TileEntry* __restrict__ tiles,
     int K, int N,                                                    // contraction length; weight rows per matrix
     void* __restrict__ out, float* __restrict__ out_scale) {
   using C = Cfg<XW>;
@@ -179,12 +176,24 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
   // deal contiguous item ranges to the 8 XCDs (workgroup ids are issued round-robin over XCDs)
-  const int n_items = hdr->n_items;
+  // work items = (row tile, column block) pairs in [expert][column block][row tile] order
+  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
+  const int n_items = hdr->n_tiles * ncb;
   const int per_xcd = (n_items + 7) >> 3;
   const int slot = blockIdx.x >> 3;
   const int item_id = (blockIdx.x & 7) * per_xcd + slot;
   if (slot >= per_xcd || item_id >= n_items) return;
-  const WorkItem item = items[item_id];
+  struct { int expert, row_start, row_count, col_block; } item;
+  {
+    const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
+    const int nt = moe_tile_count(te.rows, BM), tr = moe_tile_rows(te.rows, BM);
+    const int local = item_id - te.first_tile * ncb;
+    item.col_block = nt == 1 ? local : local / nt;
+    const int rt = local - item.col_block * nt;
+    item.expert = te.expert;
+    item.row_start = te.row_start + rt * tr;
+    item.row_count = min(tr, te.rows - rt * tr);
+  }
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -477,9 +486,10 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
 
 int col_blocks(int mode, int N) { return mode == MODE_GATEUP ? N / 128 : (N + 255) / 256; }
 
-int max_items_for(int R, int E, int n_col_blocks, int bm) {
-  long long tiles = (long long)(R + bm - 1) / bm + (E < R ? E : R);
-  return (int)(tiles * n_col_blocks);
+int max_tiles_for(int R, int E, int bm) { return (int)((long long)(R + bm - 1) / bm + (E < R ? E : R)); }
+
+TileList tile_list(void* ws, int R, int E, int bm) {
+  return TileList{max_tiles_for(R, E, bm), (TileHeader*)ws, (TileEntry*)((char*)ws + sizeof(TileHeader))};
 }
 
 template <int MODE, int XW>
@@ -487,19 +497,15 @@ int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const
                const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
                void* out, float* out_scale, void* ws, bool list_built, hipStream_t s) {
   using C = Cfg<XW>;
-  const int ncb = col_blocks(MODE, N);
-  const int max_items = max_items_for(R, E, ncb, C::BM);
-  WorkHeader* hdr = (WorkHeader*)ws;
-  WorkItem* items = (WorkItem*)((char*)ws + sizeof(WorkHeader));
-  if (!list_built) {
-    const ListSpec spec{ncb, max_items, hdr, items};
-    hipLaunchKernelGGL(build_items_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, C::BM, spec, spec);
-  }
+  const TileList l = tile_list(ws, R, E, C::BM);
+  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, C::BM, l);
   static std::atomic<unsigned long long> lds_raised{0};
   if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE, XW>, C::LDS_BYTES, lds_raised)) return rc;
-  const int grid = ((max_items + 7) / 8) * 8;
+  const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
+  MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
+  const int grid = (int)((max_items + 7) / 8) * 8;
   hipLaunchKernelGGL((grouped_gemm_kernel<MODE, XW>), dim3(grid), dim3(NT), C::LDS_BYTES, s, xq, sx, row_ids, w0, sw0,
-                     w1, sw1, hdr, items, K, N, out, out_scale);
+                     w1, sw1, l.hdr, l.tiles, K, N, out, out_scale);
   return moe_check_hip(hipGetLastError(), "gemm launch");
 }
 
@@ -544,10 +550,9 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
 }  // namespace
 
 extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
-  // enough for either GEMM: column blocks of 128 bound both; the tile height is the one the launch will choose
-  int ncb = (N_out + 127) / 128;
+  (void)N_out;   // the tile list does not depend on the number of output columns
   const int bm = tile_height(tile_config(R, E));
-  return sizeof(WorkHeader) + (size_t)max_items_for(R, E, ncb, bm < 128 ? bm : 128) * sizeof(WorkItem) + 256;
+  return sizeof(TileHeader) + (size_t)max_tiles_for(R, E, bm < 128 ? bm : 128) * sizeof(TileEntry) + 256;
 }
 
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
@@ -592,31 +597,15 @@ extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8
   return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, stream);
 }
 
-namespace {
-int list_specs(int E, int R, int D, int I, void* ws_gateup, void* ws_down, size_t ws_bytes_each, ListSpec* l0,
-               ListSpec* l1, int* bm_out) {
-  MOE_REQUIRE(ws_bytes_each >= moe_gemm_workspace_bytes(R, E, I > D ? I : D), MOE_ERR_WORKSPACE_TOO_SMALL,
-              "gemm lists: workspace too small");
-  const int bm = tile_height(tile_config(R, E));
-  const int ncb_a = col_blocks(MODE_GATEUP, I), ncb_b = col_blocks(MODE_DOWN, D);
-  *l0 = ListSpec{ncb_a, max_items_for(R, E, ncb_a, bm), (WorkHeader*)ws_gateup,
-                 (WorkItem*)((char*)ws_gateup + sizeof(WorkHeader))};
-  *l1 = ListSpec{ncb_b, max_items_for(R, E, ncb_b, bm), (WorkHeader*)ws_down,
-                 (WorkItem*)((char*)ws_down + sizeof(WorkHeader))};
-  *bm_out = bm;
-  return MOE_OK;
-}
-}  // namespace
-
-// Lists the work items of a layer's gate/up GEMM (into ws_gateup) and down GEMM (into ws_down) in one launch;
-// the *_impl entry points then take list_built = true.
-int moe_gemm_build_lists(const int32_t* group_offsets, int E, int R, int D, int I, void* ws_gateup, void* ws_down,
-                         size_t ws_bytes_each, moe_stream_t stream) {
-  ListSpec a, b;
-  int bm;
-  int rc = list_specs(E, R, D, I, ws_gateup, ws_down, ws_bytes_each, &a, &b, &bm);
-  if (rc) return rc;
+// Lists the row tiles of a layer's routed GEMMs once (gate/up and down share the list); the *_impl entry points then
+// take list_built = true with the same ws.
+int moe_gemm_build_tiles(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream) {
+  MOE_REQUIRE(group_offsets && ws, MOE_ERR_NULL, "gemm tiles: null pointer");
+  MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0, MOE_ERR_BAD_SHAPE, "gemm tiles: need 1 <= E <= 1024, got E=%d R=%d", E, R);
+  MOE_REQUIRE(ws_bytes >= moe_gemm_workspace_bytes(R, E, 0), MOE_ERR_WORKSPACE_TOO_SMALL, "gemm tiles: workspace too small");
   if (R == 0) return MOE_OK;
-  hipLaunchKernelGGL(build_items_kernel, dim3(2), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, bm, a, b);
-  return moe_check_hip(hipGetLastError(), "gemm lists launch");
+  const int bm = tile_height(tile_config(R, E));
+  hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, bm,
+                     tile_list(ws, R, E, bm));
+  return moe_check_hip(hipGetLastError(), "gemm tiles launch");
 }
