@@ -223,10 +223,13 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     rc = moe_route_sigmoid_grouped_impl(src, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
                                         a->routed_scale, idx, w, stream);
   if (rc) return join(rc);
-  if ((rc = moe_permute(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
-                        b.permute_ws_bytes, stream)))
+  // the permutation kernels also list the routed GEMMs' row tiles (they hold every expert's row range anyway)
+  TileList tiles;
+  int bm = 0;
+  if ((rc = moe_gemm_tile_list(R, a->E, b.gemm_ws, b.gemm_ws_bytes, &tiles, &bm))) return join(rc);
+  if ((rc = moe_permute_impl(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
+                             b.permute_ws_bytes, tiles, bm, stream)))
     return join(rc);
-  if ((rc = moe_gemm_build_tiles(b.group_offsets, a->E, R, b.gemm_ws, b.gemm_ws_bytes, stream))) return join(rc);
   if (!quant_joined) {
     if (rc_shared) return join(rc_shared);
     if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);

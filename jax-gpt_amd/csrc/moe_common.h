@@ -83,8 +83,13 @@ int moe_route_softmax_impl(const LogitSource& src, int M, int E, int k, int reno
 int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, int M, int E, int n_group,
                                    int topk_group, int k, int renorm, float routed_scale, int32_t* idx, float* w,
                                    moe_stream_t stream);
-// grouped GEMMs with an optional pre-built tile list in ws (moe_gemm.hip); the extern "C" entry points build their own
-int moe_gemm_build_tiles(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream);
+// grouped GEMMs with an optional pre-built tile list in ws (moe_gemm.hip); the extern "C" entry points build their
+// own.  moe_gemm_tile_list describes the list the GEMMs of (R rows, E experts) expect in ws, so that the permutation
+// kernels, which hold every expert's row range anyway, can write it (moe_permute_impl) and no launch is spent on it.
+int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list, int* bm);
+int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_sizes, int32_t* group_offsets,
+                     int32_t* sorted_token_ids, int32_t* sort_order, int32_t* inv_perm, void* ws, size_t ws_bytes,
+                     TileList tiles, int bm, moe_stream_t stream);
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
                          const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
                          int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,

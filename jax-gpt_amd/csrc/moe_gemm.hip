@@ -597,15 +597,12 @@ extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8
   return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, stream);
 }
 
-// Lists the row tiles of a layer's routed GEMMs once (gate/up and down share the list); the *_impl entry points then
-// take list_built = true with the same ws.
-int moe_gemm_build_tiles(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream) {
-  MOE_REQUIRE(group_offsets && ws, MOE_ERR_NULL, "gemm tiles: null pointer");
+// The tile list that the GEMM launches of (R rows, E experts) read from ws when they are told list_built = true.
+int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list, int* bm) {
+  MOE_REQUIRE(ws && list && bm, MOE_ERR_NULL, "gemm tiles: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0, MOE_ERR_BAD_SHAPE, "gemm tiles: need 1 <= E <= 1024, got E=%d R=%d", E, R);
   MOE_REQUIRE(ws_bytes >= moe_gemm_workspace_bytes(R, E, 0), MOE_ERR_WORKSPACE_TOO_SMALL, "gemm tiles: workspace too small");
-  if (R == 0) return MOE_OK;
-  const int bm = tile_height(tile_config(R, E));
-  hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, bm,
-                     tile_list(ws, R, E, bm));
-  return moe_check_hip(hipGetLastError(), "gemm tiles launch");
+  *bm = tile_height(tile_config(R, E));
+  *list = tile_list(ws, R, E, *bm);
+  return MOE_OK;
 }
