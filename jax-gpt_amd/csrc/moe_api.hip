@@ -199,6 +199,13 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     return moe_check_hip(e2, "forward: join");
   };
 
+  // Small batches: the quantisation is over before the caller's stream has got past the fork, so waiting for it
+  // here costs nothing, and the routed gate/up GEMM then follows the permutation without an event wait between
+  // them (each cross-stream wait costs a few microseconds of launch latency).
+  if (!quant_joined && !rc_shared && (long long)a->M * a->D <= (1ll << 21)) {
+    if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
+    quant_joined = true;
+  }
   // With a router weight the routing kernel adds the matmul's split-K partial sums itself: the (M, E) logits
   // are written only when out_logits asks for them.
   LogitSource src{a->logits, nullptr, 0, a->E, nullptr, nullptr};
