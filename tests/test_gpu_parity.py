@@ -622,3 +622,27 @@ def test_concurrent_calls_on_two_streams(jg):
         assert len(results[i]) == 20
         for out in results[i]:
             assert torch.equal(out, cases[i][5])
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_shapes_full_parity(jg, seed):
+    """Twelve random small layers per seed, both routers, with and without a shared expert (any intermediate size),
+    renormalised or not: integers bit-exact, outputs within the tolerance of helpers.assert_close_out."""
+    rng = np.random.default_rng(seed)
+    for it in range(12):
+        D = int(rng.integers(1, 9)) * 128
+        I = int(rng.integers(1, 7)) * 128
+        SI = int(rng.choice([0, 0, 128, 256, I]))
+        grouped = bool(rng.integers(0, 2))
+        if grouped:
+            G = int(rng.choice([1, 2, 4, 8])); per = int(rng.choice([1, 2, 4, 8, 16])); E = G * per
+            TG = int(rng.integers(1, G + 1)); k = int(rng.integers(1, min(8, TG * per) + 1))
+            kw = dict(routing="sigmoid_grouped", n_group=G, topk_group=TG, routed_scale=float(rng.choice([1.0, 2.5])))
+        else:
+            E = int(rng.integers(1, 65)); k = int(rng.integers(1, min(E, 8) + 1))
+            kw = dict(routing="softmax")
+        kw["renorm"] = bool(rng.integers(0, 2))
+        M = int(rng.choice([1, 2, 3, 7, 17, 33, 64, 100, 129, 257, 300, 513]))
+        _say("random layer", seed, it, M, D, E, k, I, SI, kw)
+        prob = H.make_problem(M=M, D=D, E=E, k=k, I=I, SI=SI, seed=100 * seed + it, routing=kw["routing"])
+        _run_full(jg, prob, k, **kw)
