@@ -171,6 +171,16 @@ __device__ __forceinline__ void dma4(const uint8_t* base, unsigned off, uint8_t*
   const unsigned m0v = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)l);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
 }
+// the same two copies with the LDS destination given as a 32-bit LDS address (uniform): keeps 64-bit generic
+// pointers to LDS, which the compiler holds in vector register pairs, out of the loops that issue the copies
+__device__ __forceinline__ void dma16(const uint8_t* base, unsigned off, unsigned lds_addr) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
+}
+__device__ __forceinline__ void dma4(const uint8_t* base, unsigned off, unsigned lds_addr) {
+  const unsigned m0v = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory", "m0");
+}
 __device__ __forceinline__ void wait_lgkm0() { __builtin_amdgcn_s_waitcnt(0xC07F); }   // lgkmcnt = 0, other counters untouched
 template <int N> __device__ __forceinline__ void wait_vm() {
   static_assert(N >= 0 && N < 64, "vmcnt range");

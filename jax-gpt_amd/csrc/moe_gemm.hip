@@ -208,13 +208,18 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
   const int drow = lane >> 3, dchunk = lane & 7;
   // the weight rows of one wave all come from one matrix: waves 0-3 copy gate rows, 4-7 up rows
   const uint8_t* wmat = (MODE == MODE_GATEUP && wave >= 4 ? w1 : w0) + (size_t)e * N * K;   // uniform
-  unsigned woff[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = (wave * 4 + i) * 8 + drow;                   // row within the 256-row weight tile
-    const int piece = dchunk ^ ((r >> 1) & 7);
-    const int grow = MODE == MODE_GATEUP ? wrow0 + (r & 127) : min(wrow0 + r, N - 1);
-    woff[i] = (unsigned)grow * (unsigned)K + piece * 16;       // < N*K <= 4 GB (checked by the launcher)
+  // Row group i of the wave holds tile rows 32 wave + 8 i + drow: consecutive groups are 8 weight rows apart (a
+  // uniform stride, added to the scalar base when the copy is issued) and their swizzled 16-byte piece alternates
+  // between two values, so two lane offsets serve all four groups.  A wave whose 32 rows lie past the matrix (the
+  // upper half of a last, half-filled column block) reads the last 32 rows instead; nothing of what it contributes
+  // is stored.
+  unsigned woff[2];
+  {
+    int grow = MODE == MODE_GATEUP ? wrow0 + ((wave * 32) & 127) : wrow0 + wave * 32;
+    if (MODE == MODE_DOWN && grow >= N) grow = N - 32;
+    const int piece = dchunk ^ (drow >> 1);
+    woff[0] = (unsigned)(grow + drow) * (unsigned)K + piece * 16;        // < N*K <= 4 GB (checked by the launcher)
+    woff[1] = (unsigned)(grow + drow) * (unsigned)K + (piece ^ 4) * 16;
   }
   unsigned xoff[C::X_DMA];
 #pragma unroll
@@ -243,14 +248,15 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
   // groups are a prefix of its X_DMA groups.
   const int nxv = C::XSKIP ? min(C::X_DMA, max(0, (((item.row_count + 7) >> 3) - wave + NWAVES - 1) / NWAVES)) : C::X_DMA;
   // copy operation i (0 <= i < VM_PER_STEP) of K step kb
+  const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);   // LDS address of the ring
   auto issue_op = [&](int kb, int i) {
-    uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
-    if (i < 4) dma16(wmat + (size_t)kb * BK, woff[i], st + (wave * 4 + i) * 1024);
+    const unsigned st = lds0 + (unsigned)(kb % C::NSTAGE) * C::STAGE_BYTES;
+    if (i < 4) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (wave * 4 + i) * 1024u);
     else if (i < 4 + C::X_DMA) {
       if (!C::XSKIP || i - 4 < nxv)
-        dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + ((i - 4) * NWAVES + wave) * 1024);
+        dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + ((i - 4) * NWAVES + wave) * 1024u);
     }
-    else if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4);
+    else if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4u);
   };
   auto issue = [&](int kb) {
 #pragma unroll
