@@ -1,6 +1,6 @@
 """Checkpoint ingest for the MoE layer: HuggingFace state-dict tensors -> the `params` dict of `moe_layer`.
 
-Two on-disk formats feed the kernels:
+Three on-disk formats feed the kernels:
 
 * Qwen3.5 (what the reference loads, jax_gpt/models/qwen35/weight_loader.py:42-63): bf16/f32 tensors, experts
   fused as `mlp.experts.gate_up_proj` (E, 2I, D) and `mlp.experts.down_proj` (E, D, I).  HF stores Linear
@@ -11,7 +11,10 @@ Two on-disk formats feed the kernels:
   `.weight_scale_inv` ((out/128, in/128) f32) pair per expert.  Already the kernels' number format: the tensors
   are stacked along a new expert axis and used as they are.
 
-Both return plain dicts of torch tensors on `device`; only the bf16 -> fp8 quantisation needs the GPU library.
+* Qwen3-MoE (Qwen3-30B-A3B and the like; transformers' Qwen3MoeSparseMoeBlock): bf16 `experts.{e}.{gate,up,down}_proj.weight`
+  (out, in) per expert, no shared expert; stacked along a new expert axis, then treated like the Qwen3.5 tensors.
+
+All return plain dicts of torch tensors on `device`; only the bf16 -> fp8 quantisation needs the GPU library.
 Inputs are mappings name -> torch.Tensor, e.g. `safetensors.torch.load_file(path)`.
 """
 from __future__ import annotations
@@ -113,4 +116,33 @@ def moe_params_from_block_fp8_state_dict(sd, prefix, n_experts, device="cuda"):
         "shared": shared,
         "gate_weight": _router_view(_get(sd, f"{prefix}.mlp.gate.weight"), device),
         "bias": None if bias is None else bias.to(device=device, dtype=torch.float32),
+    }
+
+
+def moe_params_from_qwen3_moe_state_dict(sd, prefix, n_experts, device="cuda", quantize=True):
+    """Qwen3-MoE layer (transformers' Qwen3MoeSparseMoeBlock): `mlp.gate.weight` (E, D) and per-expert bf16
+    `mlp.experts.{e}.{gate,up,down}_proj.weight` in (out, in) layout, no shared expert.
+
+    Returns the dict `moe_layer(x, params, k)` takes (moe.py:235; routing there is softmax top-k with
+    renormalisation, which is Qwen3-MoE's norm_topk_prob=True).  quantize as in moe_params_from_qwen35_state_dict;
+    the experts of one projection are stacked and quantised before the next projection is touched."""
+
+    def stacked(proj):
+        ws = [_get(sd, f"{prefix}.mlp.experts.{e}.{proj}.weight") for e in range(n_experts)]
+        shape = tuple(ws[0].shape)
+        for e, w in enumerate(ws):
+            if w.dim() != 2 or tuple(w.shape) != shape:
+                raise ValueError(f"{prefix}.mlp.experts.{e}.{proj}.weight: expected {shape}, got {tuple(w.shape)}")
+        w = torch.stack([w.to(device) for w in ws])                  # (E, out, in)
+        if w.dtype not in (torch.bfloat16, torch.float32):
+            w = w.to(torch.bfloat16)
+        if quantize:
+            return _moe.quantize_weight_block(w.contiguous())
+        return w.transpose(1, 2).contiguous()                         # reference layout (E, in, out)
+
+    return {
+        "gate_weight": _router_view(_get(sd, f"{prefix}.mlp.gate.weight"), device),
+        "gate_proj": stacked("gate_proj"),
+        "up_proj": stacked("up_proj"),
+        "down_proj": stacked("down_proj"),
     }

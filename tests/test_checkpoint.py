@@ -129,3 +129,49 @@ def test_block_fp8_ingest_runs_the_layer():
                         routing="sigmoid_grouped", bias=prob["bias"], n_group=4, topk_group=2)
     assert np.array_equal(dbg["indices"].cpu().numpy(), ref["indices"])
     H.assert_close_out(H.bf16_to_np(out), ref["out"], tol=1e-2, inner=128)
+
+
+def _qwen3_moe_sd(E, D, I, seed, prefix="model.layers.1"):
+    g = torch.Generator().manual_seed(seed)
+    r = lambda *s, sc=0.05: (torch.randn(*s, generator=g) * sc).to(torch.bfloat16)
+    sd = {f"{prefix}.mlp.gate.weight": r(E, D, sc=0.2)}
+    for e in range(E):
+        sd[f"{prefix}.mlp.experts.{e}.gate_proj.weight"] = r(I, D)
+        sd[f"{prefix}.mlp.experts.{e}.up_proj.weight"] = r(I, D)
+        sd[f"{prefix}.mlp.experts.{e}.down_proj.weight"] = r(D, I)
+    return sd
+
+
+def test_qwen3_moe_layouts_on_cpu():
+    """Per-expert (out, in) tensors become the reference's stacked (E, in, out) arrays; a missing expert is named."""
+    import jax_gpt_amd.checkpoint as ck
+    E, D, I = 4, 256, 128
+    sd = _qwen3_moe_sd(E, D, I, 3)
+    p = ck.moe_params_from_qwen3_moe_state_dict(sd, "model.layers.1", E, device="cpu", quantize=False)
+    assert p["gate_proj"].shape == (E, D, I) and p["down_proj"].shape == (E, I, D)
+    for e in range(E):
+        assert torch.equal(p["up_proj"][e], sd[f"model.layers.1.mlp.experts.{e}.up_proj.weight"].t())
+    assert torch.equal(p["gate_weight"], sd["model.layers.1.mlp.gate.weight"].t())
+    assert "shared_gate_proj" not in p
+    bad = dict(sd); del bad["model.layers.1.mlp.experts.2.down_proj.weight"]
+    with pytest.raises(KeyError, match="experts.2.down_proj"):
+        ck.moe_params_from_qwen3_moe_state_dict(bad, "model.layers.1", E, device="cpu", quantize=False)
+    bad = dict(sd); bad["model.layers.1.mlp.experts.1.gate_proj.weight"] = torch.zeros(I + 1, D, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="experts.1.gate_proj"):
+        ck.moe_params_from_qwen3_moe_state_dict(bad, "model.layers.1", E, device="cpu", quantize=False)
+
+
+@pytest.mark.gpu
+def test_qwen3_moe_checkpoint_runs_the_layer():
+    """Quantised at load or on first use, the layer gives the same bits; no shared expert in this family."""
+    import jax_gpt_amd as jg
+    import jax_gpt_amd.checkpoint as ck
+    E, D, I, k = 8, 256, 128, 2
+    sd = _qwen3_moe_sd(E, D, I, 4)
+    x = (torch.randn(2, 24, D, generator=torch.Generator().manual_seed(5)) * 1.0).to(torch.bfloat16).cuda()
+    pq = ck.moe_params_from_qwen3_moe_state_dict(sd, "model.layers.1", E, quantize=True)
+    pp = ck.moe_params_from_qwen3_moe_state_dict(sd, "model.layers.1", E, quantize=False)
+    out_q = jg.moe_layer(x, pq, k)
+    out_p = jg.moe_layer(x, pp, k)
+    assert out_q.shape == x.shape and torch.isfinite(out_q.float()).all()
+    assert torch.equal(out_q, out_p)
