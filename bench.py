@@ -30,12 +30,12 @@ PEAK_HBM_GBS = 8000.0        # MI355X HBM3E (published)
 MEASURED_TRAFFIC = {"deepseek_v3_prefill": 8757e6 + 146e6}
 
 WORKLOADS = {
-    # BASELINE config 3 / 4: DeepSeek-V3-style layer
+    # benchmark configs 3 and 4 (BASELINE.json): DeepSeek-V3-style layer
     "deepseek_v3_prefill": dict(M=8192, D=7168, E=256, k=8, I=2048, SI=2048, routing="sigmoid_grouped",
                                 n_group=8, topk_group=4),
     "deepseek_v3_decode": dict(M=64, D=7168, E=256, k=8, I=2048, SI=2048, routing="sigmoid_grouped",
                                n_group=8, topk_group=4),
-    # BASELINE config 2: Qwen3-MoE-style layer
+    # benchmark config 2 (BASELINE.json): Qwen3-MoE-style layer
     "qwen3_moe_prefill": dict(M=4096, D=2048, E=128, k=8, I=768, SI=0, routing="softmax", n_group=1, topk_group=1),
 }
 

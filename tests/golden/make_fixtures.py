@@ -1,4 +1,4 @@
-"""Writes tests/golden/config1_oracle.npz: the oracle's results for BASELINE config 1 (256 tokens, hidden 512,
+"""Writes tests/golden/config1_oracle.npz: the oracle's results for config 1 of BASELINE.json (256 tokens, hidden 512,
 8 experts top-2 softmax, intermediate 1024, seed 0).  The reference holds no vectors for this path and cannot run
 here (JAX is absent), so these are the oracle's own values, frozen: integer results in full, the bf16 output as a
 checksum plus a few rows.  They guard the oracle (and through it the GPU path) against silent change."""

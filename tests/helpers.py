@@ -64,7 +64,7 @@ def assert_close_out(got, want, tol=1e-2, inner=None):
         contraction shorter than 1024 after the fp8 re-quantisation the bound is tol * sqrt(1024 / inner),
         because one flipped intermediate code (below) weighs more against a shorter sum: random small
         shapes reach 1.0e-2 ... 1.15e-2 at inner = 256 / 512 in about one case in twenty (median row
-        error stays below 1e-3); every BASELINE config with inner >= 1024 is held to tol itself;
+        error stays below 1e-3); every config of BASELINE.json with inner >= 1024 is held to tol itself;
     (2) row-wise ||y - ref||_2 / ||ref||_2: mean over rows <= 0.4*tol (16 rows or more), every row
         <= tol + 0.45/sqrt(inner), where `inner` is the length of the contraction that
         follows an fp8 re-quantisation (the expert intermediate size; None = no such stage);

@@ -1,4 +1,4 @@
-"""Parity at the benchmark configurations' full sizes (BASELINE configs 2-5).
+"""Parity at the benchmark configurations' full sizes (configs 2-5 of BASELINE.json).
 
 The oracle cannot run these sizes in full, so each test checks
   * every integer result (routing indices, group sizes, permutation) exactly against

@@ -226,7 +226,7 @@ def _run_full(jg, prob, top_k, **kw):
 
 
 def test_config1_tiny_full_parity(jg):
-    """BASELINE config 1: 256 tokens, hidden 512, 8 experts top-2 softmax, intermediate 1024, seed 0."""
+    """Config 1 of BASELINE.json: 256 tokens, hidden 512, 8 experts top-2 softmax, intermediate 1024, seed 0."""
     _say("config 1")
     prob = H.make_problem(M=256, D=512, E=8, k=2, I=1024, seed=0)
     _run_full(jg, prob, 2, routing="softmax")

@@ -336,7 +336,7 @@ def test_swiglu_closed_form():
 
 def test_oracle_matches_committed_fixture_for_config1():
     """tests/golden/config1_oracle.npz (written by tests/golden/make_fixtures.py) freezes the oracle's results for
-    BASELINE config 1; the GPU tests compare against the live oracle, this keeps the oracle itself from drifting."""
+    benchmark config 1 (BASELINE.json); the GPU tests compare against the live oracle, this keeps the oracle itself from drifting."""
     import os
     from tests.golden import make_fixtures
     want = np.load(os.path.join(os.path.dirname(make_fixtures.__file__), "config1_oracle.npz"))
