@@ -107,6 +107,7 @@ def run_workload(jg, torch, name, cfg, layer, steps, warmup):
     gs = dbg["group_sizes"].cpu()
     touched = int((gs > 0).sum())
     assert int(gs.sum()) == cfg["M"] * cfg["k"]
+    log(f"{name}: rows per expert, ascending: {sorted(int(v) for v in gs)}")
     ev_ms, wall_ms = timed(torch, lambda: jg.moe_experts(x, logits, **kw), steps, warmup)
     M, D, E, k, I, SI = (cfg[n] for n in ("M", "D", "E", "k", "I", "SI"))
     R = M * k

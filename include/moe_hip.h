@@ -31,6 +31,13 @@
 extern "C" {
 #endif
 
+/* The library is built with hidden visibility: only what this header declares is exported. */
+#if defined(__GNUC__) || defined(__clang__)
+#define MOE_API __attribute__((visibility("default")))
+#else
+#define MOE_API
+#endif
+
 #define MOE_OK 0
 #define MOE_ERR_BAD_SHAPE (-1)
 #define MOE_ERR_BAD_ALIGN (-2)
@@ -43,44 +50,44 @@ extern "C" {
 
 typedef void* moe_stream_t; /* a hipStream_t */
 
-int moe_abi_version(void);
-const char* moe_last_error(void);
+MOE_API int moe_abi_version(void);
+MOE_API const char* moe_last_error(void);
 
 /* moe.py:51-53 (softmax in f32, lax.top_k, renormalise).  E <= 1024, k <= 32, k <= E. */
-int moe_route_softmax_topk(const float* logits, int M, int E, int k, int renorm,
+MOE_API int moe_route_softmax_topk(const float* logits, int M, int E, int k, int renorm,
                            int32_t* idx, float* w, moe_stream_t stream);
 
 /* DeepSeek-V3 router: sigmoid scores, +bias for selection only, group score = sum of
  * the group's top-2, keep topk_group groups, top-k among them, weights = un-biased
  * scores (renormalised with +1e-20) * routed_scale.  Replaces moe.py:37-55 for the
  * DeepSeek-shaped configs.  bias may be NULL.  E <= 1024, n_group <= 64. */
-int moe_route_sigmoid_grouped(const float* logits, const float* bias, int M, int E, int n_group,
+MOE_API int moe_route_sigmoid_grouped(const float* logits, const float* bias, int M, int E, int n_group,
                               int topk_group, int k, int renorm, float routed_scale,
                               int32_t* idx, float* w, moe_stream_t stream);
 
 /* moe.py:58-80 (_sort_and_group): stable counting sort of the flat (token, slot)
  * list by expert id.  Outputs group_sizes (E), group_offsets (E+1), sorted_token_ids
  * (R), sort_order (R), inv_perm (R); any of the last three may be NULL. */
-size_t moe_permute_workspace_bytes(int M, int k, int E);
-int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* group_sizes,
+MOE_API size_t moe_permute_workspace_bytes(int M, int k, int E);
+MOE_API int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* group_sizes,
                 int32_t* group_offsets, int32_t* sorted_token_ids, int32_t* sort_order,
                 int32_t* inv_perm, void* ws, size_t ws_bytes, moe_stream_t stream);
 
 /* 1x128 activation quantiser (replaces fp8.py:30-45's per-row quantiser):
  * scale = 448/amax, q = e4m3(clamp(x*scale)), sx = 1/scale.  K % 128 == 0. */
-int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream);
+MOE_API int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream);
 
 /* 128x128 weight block quantiser (replaces quantize.py:18-42's per-row quantiser;
  * layout (E, out, in) as quantize.py:31-35).  src_is_f32: 0 = bf16 source, 1 = f32. */
-int moe_quant_weight_block(const void* w, int src_is_f32, int E, int N, int K, uint8_t* wq,
+MOE_API int moe_quant_weight_block(const void* w, int src_is_f32, int E, int N, int K, uint8_t* wq,
                            float* sw, moe_stream_t stream);
 
 /* moe.py:85-86 + silu*mul of :87, fused: for rows [group_offsets[e], group_offsets[e+1])
  * h = silu(x . Wgate[e]^T) * (x . Wup[e]^T), then 1x128 fp8 quantisation of h.
  * row_ids (R) maps sorted position -> row of xq/sx (the gather of moe.py:79 without
  * materialising x_sorted); NULL = identity (pre-dispatched rows).  D, I % 128 == 0. */
-size_t moe_gemm_workspace_bytes(int R, int E, int N_out);
-int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+MOE_API size_t moe_gemm_workspace_bytes(int R, int E, int N_out);
+MOE_API int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
                                const uint8_t* w_gate, const float* sw_gate,
                                const uint8_t* w_up, const float* sw_up,
                                const int32_t* group_offsets, int E, int R, int D, int I,
@@ -88,7 +95,7 @@ int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t
                                moe_stream_t stream);
 
 /* moe.py:87 (the third ragged_dot): y = h . Wdown[e]^T, bf16 out (R, D). */
-int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
+MOE_API int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
                       const float* sw_down, const int32_t* group_offsets, int E, int R, int I,
                       int D, void* y_bf16, void* ws, size_t ws_bytes, moe_stream_t stream);
 
@@ -97,7 +104,7 @@ int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
  * NULL (moe.py:281 adds the shared expert's output); shared_gate may be NULL (= 1; moe.py:278-279
  * multiplies the shared expert's output by sigmoid(x @ shared_expert_gate_weight)); residual
  * (M, D) bf16 or NULL is the layer's input added last (x = x + moe_out, block.py:58 and :91). */
-int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
+MOE_API int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
                 const void* shared_bf16, const float* shared_gate, const void* residual_bf16, int M, int k,
                 int D, void* out_bf16, moe_stream_t stream);
 
@@ -106,8 +113,8 @@ int moe_combine(const void* y_bf16, const float* w, const int32_t* inv_perm,
  * checkpoint layout of mlp.gate.weight; the reference's in-memory array is its transpose (D, E));
  * w_shared_gate is (1, D) bf16 or NULL.  logits (M, E) f32 hold bf16-rounded values; shared_gate
  * (M) f32 holds bf16-rounded sigmoids (NULL iff w_shared_gate is NULL). */
-size_t moe_router_workspace_bytes(int M, int D, int E);
-int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
+MOE_API size_t moe_router_workspace_bytes(int M, int D, int E);
+MOE_API int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
                       const void* w_shared_gate_bf16, float* logits, float* shared_gate, void* ws,
                       size_t ws_bytes, moe_stream_t stream);
 
@@ -115,7 +122,7 @@ int moe_router_logits(const void* x_bf16, int M, int D, const void* w_router_bf1
  * bf16) as called in front of the MoE layer (block.py:54, :88), fused with the 1x128 quantisation of the
  * normalised row.  weight (D) f32; normed_bf16 (M, D) may be NULL when only the fp8 form is needed.
  * D <= 8192. */
-int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
+MOE_API int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
                       uint8_t* xq, float* sx, moe_stream_t stream);
 
 /* The whole path (moe.py:97-114 + 225-232 + 281): router logits in, combined hidden
@@ -141,6 +148,8 @@ typedef struct MoeForwardArgs {
   int32_t* out_group_sizes;      /* (E) */
   int32_t* out_sorted_token_ids; /* (R) */
   int32_t* out_inv_perm;         /* (R) */
+  uint8_t* out_hq;               /* (R, I) e4m3 codes of the SwiGLU output, rows in sorted order */
+  float* out_sh;                 /* (R, I/128) their 1x128 scales */
   /* router in front of the path (NULL = the caller supplies logits) */
   const void* w_router;          /* (E, D) bf16: logits = bf16(x . w_router^T), moe.py:50 */
   const void* w_shared_gate;     /* (1, D) bf16 or NULL: shared expert's output is scaled by
@@ -152,8 +161,8 @@ typedef struct MoeForwardArgs {
   int add_residual;              /* out = x + moe_out, added in f32 before the one bf16 rounding */
 } MoeForwardArgs;
 
-size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI);
-int moe_forward(const MoeForwardArgs* args, void* ws, size_t ws_bytes, moe_stream_t stream);
+MOE_API size_t moe_forward_workspace_bytes(int M, int D, int E, int k, int I, int SI);
+MOE_API int moe_forward(const MoeForwardArgs* args, void* ws, size_t ws_bytes, moe_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -19,6 +19,7 @@ SOURCES = ["moe_api.hip", "moe_route.hip", "moe_router.hip", "moe_permute.hip", 
            "moe_combine.hip"]
 # no v_pk_*_f32 code generation (some packed-f32 forms misbehave on this hardware pool)
 COMMON = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
+          "-fvisibility=hidden",    # only the functions include/moe_hip.h declares (MOE_API) are exported
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
           "-I", os.path.join(ROOT, "include"), "-I", CSRC]
 # routing and combine promise individually rounded f32 operations (bit-reproducible on a CPU)

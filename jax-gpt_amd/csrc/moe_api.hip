@@ -24,7 +24,7 @@ int moe_check_hip(hipError_t e, const char* what) {
   return moe_set_error(MOE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-extern "C" int moe_abi_version(void) { return 2; }
+extern "C" int moe_abi_version(void) { return 3; }
 extern "C" const char* moe_last_error(void) { return g_err; }
 
 namespace {
@@ -145,6 +145,11 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   int32_t* gsz = a->out_group_sizes ? a->out_group_sizes : b.group_sizes;
   int32_t* stid = a->out_sorted_token_ids ? a->out_sorted_token_ids : b.sorted_token_ids;
   int32_t* inv = a->out_inv_perm ? a->out_inv_perm : b.inv_perm;
+  // the intermediate h is written straight into the caller's debug arrays when both are given
+  MOE_REQUIRE((a->out_hq == nullptr) == (a->out_sh == nullptr), MOE_ERR_NULL, "forward: out_hq and out_sh come together");
+  MOE_REQUIRE(MOE_ALIGNED16(a->out_hq), MOE_ERR_BAD_ALIGN, "forward: out_hq must be 16-byte aligned");
+  uint8_t* hq = a->out_hq ? a->out_hq : b.hq;
+  float* sh = a->out_sh ? a->out_sh : b.sh;
   const int R = a->M * a->k;
   hipStream_t main_s = (hipStream_t)stream;
   MOE_REQUIRE(a->routing == MOE_ROUTING_SOFTMAX || a->routing == MOE_ROUTING_SIGMOID_GROUPED, MOE_ERR_BAD_SHAPE,
@@ -242,9 +247,9 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
   }
   if ((rc = moe_gemm_gateup_impl(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets, a->E, R,
-                                 a->D, a->I, b.hq, b.sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
+                                 a->D, a->I, hq, sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);
-  if ((rc = moe_gemm_down_impl(b.hq, b.sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
+  if ((rc = moe_gemm_down_impl(hq, sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
                                b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;

@@ -138,12 +138,23 @@ int choose_splits(int M, int N, int D) {
   return (int)s;
 }
 
+// K slices that hold at least one K step, and the bytes of their partial sums [slices][M][N]
+int slices_used(int M, int N, int D, int* k_per_split) {
+  const int splits = choose_splits(M, N, D);
+  const int kps = ((D / RBK + splits - 1) / splits) * RBK;
+  if (k_per_split) *k_per_split = kps;
+  return (D + kps - 1) / kps;
+}
+size_t partial_bytes(int M, int N, int D) { return (size_t)slices_used(M, N, D, nullptr) * (size_t)M * N * sizeof(float); }
+
 }  // namespace
 
 extern "C" size_t moe_router_workspace_bytes(int M, int D, int E) {
   if (M < 0 || D <= 0 || E <= 0) return 0;
-  const int N = E + 1;
-  return (size_t)choose_splits(M, N, D) * (size_t)M * N * sizeof(float) + 256;
+  // With or without the shared expert's gate column: without it N = E can fill one column tile fewer, and the K
+  // split chosen for the smaller grid is then deeper, so neither case bounds the other.
+  const size_t a = partial_bytes(M, E, D), b = partial_bytes(M, E + 1, D);
+  return (a > b ? a : b) + 256;
 }
 
 // The matmul alone: split-K partial sums [splits][M][N] at the start of ws (N = E, + 1 with the gate column).
@@ -159,9 +170,10 @@ int moe_router_partials(const void* x_bf16, int M, int D, const void* w_router_b
   MOE_REQUIRE(ws_bytes >= moe_router_workspace_bytes(M, D, E), MOE_ERR_WORKSPACE_TOO_SMALL,
               "router: workspace %zu < %zu", ws_bytes, moe_router_workspace_bytes(M, D, E));
   const int N = E + (w_shared_gate_bf16 ? 1 : 0);
-  const int splits = choose_splits(M, N, D);
-  const int k_per_split = ((D / RBK + splits - 1) / splits) * RBK;
-  const int used = (D + k_per_split - 1) / k_per_split;   // slices that hold at least one K step
+  int k_per_split = 0;
+  const int used = slices_used(M, N, D, &k_per_split);
+  MOE_REQUIRE(ws_bytes >= (size_t)used * (size_t)M * N * sizeof(float), MOE_ERR_WORKSPACE_TOO_SMALL,
+              "router: %d slices of %d x %d partial sums do not fit the workspace (%zu bytes)", used, M, N, ws_bytes);
   *splits_used = used;
   *n_cols = N;
   if (M == 0) return MOE_OK;

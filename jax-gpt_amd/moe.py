@@ -359,7 +359,8 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     router_logits=None); `shared_expert_gate_weight` (D, 1) then scales the shared
     expert's output by its sigmoid gate (moe.py:278-279).  `norm_weight` (D,) puts the
     block's RMSNorm in front (block.py:54) and `add_residual` its `x + moe_out` behind (:58).
-    Returns (M, D) bf16, plus a dict of the integer intermediates if return_debug."""
+    Returns (M, D) bf16, plus, if return_debug, a dict of the integer intermediates and of the quantised
+    SwiGLU output the down GEMM consumed (`hq` (R, I) e4m3 codes as uint8 and `sh` (R, I/128), sorted order)."""
     x = _dev(x, torch.bfloat16, "x")
     wr = wsg = None
     if gate_weight is not None:
@@ -433,7 +434,9 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
         R = M * top_k
         dbg = dict(indices=_empty((M, top_k), torch.int32, x), weights=_empty((M, top_k), torch.float32, x),
                    group_sizes=_empty((E,), torch.int32, x), sorted_token_ids=_empty((R,), torch.int32, x),
-                   inv_perm=_empty((R,), torch.int32, x))
+                   inv_perm=_empty((R,), torch.int32, x),
+                   hq=_empty((R, I), torch.uint8, x), sh=_empty((R, I // 128), torch.float32, x))
+        a.out_hq, a.out_sh = dbg["hq"].data_ptr(), dbg["sh"].data_ptr()
         if wr is not None:
             dbg["logits"] = _empty((M, E), torch.float32, x)
             a.out_logits = dbg["logits"].data_ptr()

@@ -32,7 +32,37 @@ def test_header_and_library_agree(dll):
     for name in declared:
         assert hasattr(dll, name), f"{name} is declared in moe_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == declared
-    assert dll.moe_abi_version() == 2
+    assert dll.moe_abi_version() == 3
+
+
+def test_library_exports_exactly_the_header(dll):
+    """Built with hidden visibility: the dynamic symbol table holds the header's functions and no internal ones."""
+    import subprocess
+    from jax_gpt_amd import _lib
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    exported = sorted(ln.split()[-1] for ln in out.splitlines() if ln.split()[-2:-1] == ["T"])
+    assert exported == _declared_functions(), set(exported) ^ set(_declared_functions())
+
+
+def test_router_workspace_covers_both_column_counts(dll):
+    """moe_router_workspace_bytes must cover the launch with and without the shared expert's gate column: when E
+    is a multiple of 128 the gate-less launch has one column tile fewer and may split K more deeply.  The library
+    checks the bytes a launch will write against ws_bytes on the host, before any GPU call: with the advertised
+    size no shape may come back as MOE_ERR_WORKSPACE_TOO_SMALL (-3); without a GPU the call then ends with
+    MOE_ERR_HIP (-4), with one it would launch, so this runs only where no GPU is present."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("host-side sizing check; runs on the CPU-only host")
+    one = C.c_void_p(256)
+    for E in (8, 128, 256, 384, 512, 1024):
+        for D in (128, 1024, 2048, 4096, 7168):
+            for M in (1, 64, 512, 2048, 4096, 8192):
+                need = dll.moe_router_workspace_bytes(M, D, E)
+                for gate in (None, one):
+                    rc = dll.moe_router_logits(one, M, D, one, E, gate, one, gate, one, need, None)
+                    assert rc != -3, (E, D, M, gate is not None, dll.moe_last_error())
+    # and a buffer sized for the smaller of the two cases is refused for the larger one (E=128, D=2048, M=4096)
+    assert dll.moe_router_logits(one, 4096, 2048, one, 128, None, one, None, one, 17_000_000, None) == -3
 
 
 def test_forward_args_struct_matches_header(dll):
