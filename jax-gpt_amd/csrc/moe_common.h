@@ -50,20 +50,27 @@ struct TileList {
   TileHeader* hdr;
   TileEntry* tiles;
 };
-// An expert with `rows` rows gets ceil(rows / bm) row tiles of equal height (a multiple of 16, the last one
-// shorter): tiles that share a weight slab then take the same time per K step and walk it together, so the
-// second reader finds it in L2.
-// (integer division costs some forty instructions on this hardware: the one-tile case takes none)
-__host__ __device__ inline int moe_tile_rows(int rows, int bm) {
-  if (rows <= bm) return bm;
-  const int t = (rows + bm - 1) / bm;
-  return ((rows + t - 1) / t + 15) & ~15;
-}
+// An expert with `rows` rows gets ceil(rows / bm) row tiles (bm = 32 or 256) whose heights, counted in units of 32
+// rows (16 for bm = 32), differ by at most one: no tile computes more than one unit of padding, and tiles that
+// share a weight slab take about the same time per K step and walk it together, so the later reader finds it in L2.
 __host__ __device__ inline int moe_tile_count(int rows, int bm) {
   if (rows <= 0) return 0;
-  if (rows <= bm) return 1;
-  const int tr = moe_tile_rows(rows, bm);
-  return (rows + tr - 1) / tr;
+  return bm == 256 ? (rows + 255) >> 8 : (rows + 31) >> 5;
+}
+// first row (relative to the expert's first) and row count of tile t of nt
+__host__ __device__ inline void moe_tile_span(int rows, int bm, int nt, int t, int& start, int& count) {
+  if (nt == 1) {   // (integer division costs some forty instructions on this hardware: the one-tile case takes none)
+    start = 0;
+    count = rows;
+    return;
+  }
+  const int ushift = bm == 256 ? 5 : 4;
+  const int units = (rows + (1 << ushift) - 1) >> ushift;
+  const int base = units / nt, extra = units - base * nt;
+  const int u0 = t * base + (t < extra ? t : extra);
+  start = u0 << ushift;
+  const int full = (base + (t < extra ? 1 : 0)) << ushift;
+  count = full < rows - start ? full : rows - start;
 }
 // Where the routing kernels take a token's logits from: an (M, E) array, or the router matmul's split-K partial
 // sums [splits][M][N] (N = E, + 1 when the shared expert's gate is the last column), which they add in slice order

@@ -148,6 +148,16 @@ struct Cfg {
 #ifndef MOE_SCHED2
 #define MOE_SCHED2 2
 #endif
+#ifndef MOE_FENCE
+#define MOE_FENCE 1
+#endif
+#ifndef MOE_ROTC
+#define MOE_ROTC 2   // MFMA groups by which wave set 1 trails wave set 0 in the tile-class kernel
+#endif
+// development ablations (results are wrong on purpose; timing only)
+#ifndef MOE_ABL
+#define MOE_ABL 0   // bit 0: no copies in the K loop, bit 1: no barrier, bit 2: copies re-read K step 0, bit 3: no FMAs, bit 4: weight copies only, bit 5: activation copies only
+#endif
 template <int XW> struct Sched {
   static constexpr int first(int j) {
     constexpr int n = Cfg<XW>::VM_PER_STEP, g = Cfg<XW>::XF;
@@ -186,13 +196,15 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
   struct { int expert, row_start, row_count, col_block; } item;
   {
     const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
-    const int nt = moe_tile_count(te.rows, BM), tr = moe_tile_rows(te.rows, BM);
+    const int nt = moe_tile_count(te.rows, BM);
     const int local = item_id - te.first_tile * ncb;
     item.col_block = nt == 1 ? local : local / nt;
     const int rt = local - item.col_block * nt;
     item.expert = te.expert;
-    item.row_start = te.row_start + rt * tr;
-    item.row_count = min(tr, te.rows - rt * tr);
+    int t0, tn;
+    moe_tile_span(te.rows, BM, nt, rt, t0, tn);
+    item.row_start = te.row_start + t0;
+    item.row_count = tn;
   }
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -490,6 +502,417 @@ __global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
   }
 }
 
+// ---- tile-class kernel ---------------------------------------------------------------------------------------
+//
+// One launch, row tiles of every height.  A work item's row tile (at most 256 rows, equal-height cuts of its
+// expert) is served by the smallest of eight compiled tile classes that holds it -- 32 XF rows, XF = 1 .. 8 MFMA
+// groups per wave and K step -- each a branch-free, fully unrolled K loop of its own with its own LDS ring: the
+// short classes have short activation tiles and use the room for more stages (160 rows and more: two stages,
+// copies one K step ahead; 64 to 128 rows: three stages, two steps ahead; 32 rows: four stages, three steps
+// ahead), because an item of a few rows only streams its 256 weight rows and lives on the bytes it keeps in
+// flight.  Rows past the end of a tile are multiplied like the others (their copies re-read the tile's last
+// row) and never stored.
+//
+// K step of a wave: XF groups; group j = its four weight fragments against activation fragment j (4 MFMAs, results
+// in p[0..3]).  The 16 FMAs that scale group j's results into the accumulators are issued between the MFMAs of
+// group j + 1 -- FMA quadruple f just before MFMA f, which overwrites p[f] -- so the matrix core works on the next
+// group while the vector ALU finishes the last one, with one set of result registers.  The last group of a step is
+// finished behind the next step's barrier, while that step's first fragments travel from LDS.
+template <int XF> struct Cls {
+  static constexpr int BM = 32 * XF, HALF = BM / 2;
+  static constexpr int STAGE_X_OFF = W_TILE_BYTES;
+  static constexpr int STAGE_S_OFF = W_TILE_BYTES + BM * BK;
+  // + 256: every wave copies 64 scale slots from its first one on (no lane mask, which would cut the unrolled K
+  // step into blocks); the surplus lanes rewrite the next waves' slots with the same values or land in this pad
+  static constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4 + 256;
+  static constexpr int NSTAGE = XF >= 5 ? 2 : XF >= 2 ? 3 : 4;
+  static constexpr int PRE = NSTAGE - 1;
+  static constexpr int X_GROUPS = 4 * XF;              // 1 KB activation row groups (8 rows) of the tile
+  static constexpr int X_OPS = (X_GROUPS + 7) / 8;     // copies per wave and step; where the groups do not fill the
+                                                       // last round, waves 4-7 repeat the copies of waves 0-3
+  static constexpr int OPS = 4 + X_OPS + 1;            // + 4 weight row groups + 1 scale copy
+  static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
+  // copy operations issued after group g: spread over the first SPREAD groups of the step
+  static constexpr int SPREAD = XF >= 6 ? XF / 2 : XF >= 3 ? 3 : XF;
+  static constexpr int first(int g) { return g <= 0 ? 0 : g >= SPREAD ? OPS : (OPS * g) / SPREAD; }
+};
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+constexpr int CLS_RING = cmax(cmax(cmax(Cls<8>::RING_BYTES, Cls<7>::RING_BYTES), cmax(Cls<6>::RING_BYTES, Cls<5>::RING_BYTES)),
+                              cmax(cmax(Cls<4>::RING_BYTES, Cls<3>::RING_BYTES), cmax(Cls<2>::RING_BYTES, Cls<1>::RING_BYTES)));
+constexpr int CLS_WSCALE_OFF = CLS_RING;                       // [2][MAX_KB] weight block scales of the work item
+constexpr int CLS_LDS_BYTES = CLS_RING + 2 * MAX_KB * 4;      // 151040; the epilogues stage through the ring (<= 128 KB)
+static_assert(CLS_LDS_BYTES <= 160 * 1024, "LDS");
+
+struct Item { int expert, row_start, row_count, col_block; };
+
+template <int MODE, int XF>
+__device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const uint8_t* __restrict__ xq,
+                                          const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
+                                          const uint8_t* __restrict__ w0, const float* __restrict__ sw0,
+                                          const uint8_t* __restrict__ w1, const float* __restrict__ sw1, int K, int N,
+                                          void* __restrict__ out, float* __restrict__ out_scale) {
+  using C = Cls<XF>;
+  constexpr int BM = C::BM, HALF = C::HALF;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wi = wave & 3, xj = wave >> 2;
+  const int fr = lane & 15, fq = lane >> 4;
+  const int KB = K / BK;
+  const int e = item.expert;
+  const int wrow0 = MODE == MODE_GATEUP ? item.col_block * 128 : item.col_block * 256;
+
+  // ---- copy sources (as in grouped_gemm_kernel): wave w fills weight row groups [4w, 4w+4), activation row
+  // groups w, w + 8, ... and 4 XF scale slots
+  const int drow = lane >> 3, dchunk = lane & 7;
+  const uint8_t* wmat = (MODE == MODE_GATEUP && wave >= 4 ? w1 : w0) + (size_t)e * N * K;   // uniform
+  unsigned woff[2];
+  {
+    int grow = MODE == MODE_GATEUP ? wrow0 + ((wave * 32) & 127) : wrow0 + wave * 32;
+    if (MODE == MODE_DOWN && grow >= N) grow = N - 32;
+    const int piece = dchunk ^ (drow >> 1);
+    woff[0] = (unsigned)(grow + drow) * (unsigned)K + piece * 16;
+    woff[1] = (unsigned)(grow + drow) * (unsigned)K + (piece ^ 4) * 16;
+  }
+  unsigned xoff[C::X_OPS];
+#pragma unroll
+  for (int i = 0; i < C::X_OPS; ++i) {
+    int grp = i * NWAVES + wave;
+    if (grp >= C::X_GROUPS) grp -= 4;
+    const int r = grp * 8 + drow;                              // row within the activation tile
+    const int piece = dchunk ^ ((r >> 1) & 7);
+    int g = item.row_start + min(r, item.row_count - 1);
+    if (row_ids) g = row_ids[g];
+    xoff[i] = (unsigned)g * (unsigned)K + piece * 16;
+  }
+  unsigned soff;
+  {
+    const int p = min(wave * (BM / 8) + lane, BM - 1);   // slots past the tile land in the pad
+    const int q = p % HALF;
+    const int r = 16 * (2 * (q % XF) + p / HALF) + q / XF;
+    int g = item.row_start + min(r, item.row_count - 1);
+    if (row_ids) g = row_ids[g];
+    soff = (unsigned)g * (unsigned)KB * 4u;
+  }
+  const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);
+  auto issue_op = [&](int kb, int i) {
+    const unsigned st = lds0 + (unsigned)(kb % C::NSTAGE) * C::STAGE_BYTES;
+    if ((MOE_ABL & 16) && i >= 4) return;
+    if ((MOE_ABL & 32) && i < 4) return;
+    if (MOE_ABL & 4) kb = 0;
+    if (i < 4) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (wave * 4 + i) * 1024u);
+    else if (i < 4 + C::X_OPS) {
+      int grp = (i - 4) * NWAVES + wave;
+      if (grp >= C::X_GROUPS) grp -= 4;
+      dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + grp * 1024u);
+    } else dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4u);
+  };
+#pragma unroll
+  for (int s = 0; s < C::PRE; ++s)
+    if (s < KB) {
+#pragma unroll
+      for (int i = 0; i < C::OPS; ++i) issue_op(s, i);
+    }
+
+  float* wscale = (float*)(lds + CLS_WSCALE_OFF);
+  for (int i = tid; i < 2 * KB; i += NT) {
+    const int h = i >= KB, kk = h ? i - KB : i;
+    float v;
+    if (MODE == MODE_GATEUP) v = (h ? sw1 : sw0)[((size_t)e * (N / 128) + item.col_block) * KB + kk];
+    else v = sw0[((size_t)e * (N / 128) + min(item.col_block * 2 + h, N / 128 - 1)) * KB + kk];
+    wscale[h * MAX_KB + kk] = v;
+  }
+  const float* ws0 = wscale + (MODE == MODE_GATEUP ? 0 : (wi >> 1) * MAX_KB);
+  const float* ws1 = wscale + MAX_KB;   // GATEUP only
+  __syncthreads();   // (the compiler waits here for the scale loads, and with them for the copies issued above)
+
+  const int lane_off0 = fr * BK + ((fq ^ (fr >> 1)) << 4);         // K bytes [16 fq, +16)
+  const int lane_off1 = fr * BK + (((fq + 4) ^ (fr >> 1)) << 4);   // K bytes [64 + 16 fq, +16)
+  int wfrag_off[4];
+#pragma unroll
+  for (int f = 0; f < 4; ++f)
+    wfrag_off[f] = (MODE == MODE_GATEUP ? ((f >> 1) * 128 + wi * 32 + (f & 1) * 16) : (wi * 64 + f * 16)) * BK;
+  auto read_frag = [&](const uint8_t* base) {
+    const v4i lo = *(const v4i*)(base + lane_off0);
+    const v4i hi = *(const v4i*)(base + lane_off1);
+    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+  };
+
+  v4f acc[4][XF];
+#pragma unroll
+  for (int f = 0; f < 4; ++f)
+#pragma unroll
+    for (int j = 0; j < XF; ++j) acc[f][j] = (v4f){0.f, 0.f, 0.f, 0.f};
+  v8i wf[4];
+  v4f p[4];
+  float pc0 = 0.f, pc1 = 0.f;   // scales of the group whose FMAs are pending
+  auto fm = [&](int f, int jj, float c0, float c1) {
+    if (!(MOE_ABL & 8)) acc[f][jj] += p[f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
+  };
+  auto mm = [&](int f, const v8i& x) {
+    p[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], x, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
+  };
+  auto fence = [&]() {
+    if (MOE_FENCE) __builtin_amdgcn_sched_barrier(0);
+  };
+  // The two waves of a SIMD belong to different wave sets (xj = 0 / 1).  Set 1 runs ROT groups behind set 0: it
+  // carries the last ROT activation fragments of a step (and their scales) in registers across the barrier and
+  // multiplies them, against the previous step's weights, first thing behind it -- so one wave of each SIMD has
+  // matrix work in registers while the other waits for its first fragments from LDS.
+  auto run = [&](auto rot_c) {
+    constexpr int ROT = decltype(rot_c)::value;
+    constexpr int NG = XF - ROT;   // groups of the current step done before the next barrier
+    constexpr int NH = ROT > 0 ? ROT : 1;
+    v8i held[NH];
+    float hc0[NH], hc1[NH];
+    auto step = [&](int kb, auto first_c, auto copy_c) {
+      constexpr bool FIRST = decltype(first_c)::value, COPY = decltype(copy_c)::value;
+      // stage kb has landed once only the copies of younger steps are outstanding
+      if (COPY || C::PRE == 1) {
+        wait_vm<(C::PRE - 1) * C::OPS>();   // (COPY steps: steps kb+1 .. kb+PRE-1 are in flight)
+      } else {
+        const int rem = KB - 1 - kb;        // the last steps: fewer and fewer copies are in flight
+        if (C::PRE > 2 && rem >= 2) wait_vm<(C::PRE > 2 ? 2 : 0) * C::OPS>();
+        else if (rem >= 1) wait_vm<C::OPS>();
+        else wait_vm<0>();
+      }
+      if (ROT > 0) wait_lgkm0();      // this wave's reads of stage kb - 1 are done before anyone overwrites it
+      if (!(MOE_ABL & 2)) __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; every wave is done with stage kb - 1
+      if constexpr (ROT > 0) {        // groups NG .. XF-1 of the previous step: held fragments, the previous weights
+        if (!FIRST) {
+#pragma unroll
+          for (int i = 0; i < ROT; ++i) {
+#pragma unroll
+            for (int f = 0; f < 4; ++f) {
+              fm(f, NG + i - 1, pc0, pc1);
+              mm(f, held[i]);
+            }
+            pc0 = hc0[i];
+            pc1 = hc1[i];
+            if (COPY && !(MOE_ABL & 1)) {
+#pragma unroll
+              for (int o = C::first(i); o < C::first(i + 1); ++o) issue_op(kb + C::PRE, o);
+            }
+            fence();
+          }
+        } else if (COPY && !(MOE_ABL & 1)) {
+#pragma unroll
+          for (int o = 0; o < C::first(ROT); ++o) issue_op(kb + C::PRE, o);
+        }
+      }
+      const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
+      const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
+      const uint8_t* xt = st + C::STAGE_X_OFF + xj * 16 * BK;
+      // finish the previous step's last group first: its FMAs need the last MFMAs' results, and those MFMAs
+      // are still reading the weight fragments that the reads below overwrite
+      if (!FIRST) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) fm(f, XF - 1, pc0, pc1);
+      }
+#pragma unroll
+      for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
+      float sxv[XF];
+      {
+        const uint8_t* sp = st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4;
+        if constexpr (XF % 4 == 0) {
+#pragma unroll
+          for (int j = 0; j < XF; j += 4) {
+            const v4f a = *(const v4f*)(sp + j * 4);
+            sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
+          }
+        } else if constexpr (XF % 2 == 0) {
+#pragma unroll
+          for (int j = 0; j < XF; j += 2) {
+            const float2 a = *(const float2*)(sp + j * 4);
+            sxv[j] = a.x; sxv[j + 1] = a.y;
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < XF; ++j) sxv[j] = *(const float*)(sp + j * 4);
+        }
+      }
+      v8i xf[2];
+      xf[0] = read_frag(xt);
+      fence();
+#pragma unroll
+      for (int j = 0; j < NG; ++j) {
+        if (j + 1 < NG) xf[(j + 1) & 1] = read_frag(xt + (j + 1) * 32 * BK);
+        if (ROT > 0 && j == 0) {
+#pragma unroll
+          for (int i = 0; i < ROT; ++i) {
+            held[i] = read_frag(xt + (NG + i) * 32 * BK);
+            hc0[i] = sxv[NG + i] * s0;
+            hc1[i] = sxv[NG + i] * s1;
+          }
+        }
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+          if (j > 0) fm(f, j - 1, pc0, pc1);
+          mm(f, xf[j & 1]);
+        }
+        pc0 = sxv[j] * s0;
+        pc1 = sxv[j] * s1;
+        if (COPY && !(MOE_ABL & 1)) {
+#pragma unroll
+          for (int o = C::first(ROT + j); o < C::first(ROT + j + 1); ++o) issue_op(kb + C::PRE, o);
+        }
+        fence();
+      }
+    };
+    constexpr std::true_type yes{};
+    constexpr std::false_type no{};
+    const int n_copy = KB - C::PRE;   // steps 0 .. n_copy-1 issue copies
+    if (n_copy > 0) step(0, yes, yes);
+    else step(0, yes, no);
+    int kb = 1;
+    for (; kb < n_copy; ++kb) step(kb, no, yes);
+    for (; kb < KB; ++kb) step(kb, no, no);
+    if constexpr (ROT > 0) {   // the groups carried out of the last step
+#pragma unroll
+      for (int i = 0; i < ROT; ++i) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+          fm(f, NG + i - 1, pc0, pc1);
+          mm(f, held[i]);
+        }
+        pc0 = hc0[i];
+        pc1 = hc1[i];
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < 4; ++f) fm(f, XF - 1, pc0, pc1);
+  };
+  constexpr int ROTC = XF >= 3 ? MOE_ROTC : XF - 1;   // (fewer groups than that: what there is)
+  if (ROTC == 0 || xj == 0) run(std::integral_constant<int, 0>{});
+  else run(std::integral_constant<int, ROTC>{});
+  __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
+
+  // ---- epilogue.  Lane holds, for fragment (f, j): tile row (2j + xj)*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
+  if (MODE == MODE_GATEUP) {
+    float* amax_s = (float*)lds;                       // [4 weight-wave groups][BM rows]
+    uint8_t* tile = lds + 4 * BM * sizeof(float);      // [BM rows][128 B], swizzled
+#pragma unroll
+    for (int j = 0; j < XF; ++j) {
+      float m = 0.f;
+#pragma unroll
+      for (int f = 0; f < 2; ++f)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float g = acc[f][j][r], u = acc[f + 2][j][r];
+          float h = g / (1.0f + __expf(-g)) * u;
+          acc[f][j][r] = h;
+          m = fmaxf(m, fabsf(h));
+        }
+      m = fmaxf(m, __shfl_xor(m, 16, MOE_WAVE));
+      m = fmaxf(m, __shfl_xor(m, 32, MOE_WAVE));
+      if (fq == 0) amax_s[wi * BM + (2 * j + xj) * 16 + fr] = m;
+    }
+    __syncthreads();
+    const int I = N;
+    uint8_t* hq = (uint8_t*)out;
+#pragma unroll
+    for (int j = 0; j < XF; ++j) {
+      const int xr = (2 * j + xj) * 16 + fr;
+      float m = fmaxf(fmaxf(amax_s[xr], amax_s[BM + xr]), fmaxf(amax_s[2 * BM + xr], amax_s[3 * BM + xr]));
+      float scale, scale_inv;
+      fp8_scales(m, scale, scale_inv);
+#pragma unroll
+      for (int f = 0; f < 2; ++f) {
+        unsigned q = pack4_e4m3(acc[f][j][0] * scale, acc[f][j][1] * scale, acc[f][j][2] * scale, acc[f][j][3] * scale);
+        const int col = wi * 32 + f * 16 + fq * 4;  // byte column within the 128-wide slab
+        *(unsigned*)(tile + swz(xr, col >> 4) + (col & 15)) = q;
+      }
+      if (wi == 0 && fq == 0 && xr < item.row_count)
+        out_scale[(size_t)(item.row_start + xr) * (I / 128) + item.col_block] = scale_inv;
+    }
+    __syncthreads();
+    const int ld_chunk = tid & 7, ld_row = tid >> 3;   // 64 rows per pass
+#pragma unroll
+    for (int i = 0; i < (BM + 63) / 64; ++i) {
+      const int r = ld_row + 64 * i;
+      if (r < item.row_count) {
+        v4i v = *(const v4i*)(tile + swz(r, ld_chunk));
+        *(v4i*)(hq + (size_t)(item.row_start + r) * I + item.col_block * 128 + ld_chunk * 16) = v;
+      }
+    }
+  } else {
+    // bf16 tile [BM rows][256 cols] = 512 B per row, 32 chunks of 16 B, swizzled with (row & 7)
+    uint8_t* tile = lds;
+#pragma unroll
+    for (int j = 0; j < XF; ++j) {
+      const int xr = (2 * j + xj) * 16 + fr;
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        const int col = wi * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
+        uint2 v;
+        v.x = (unsigned)f32_to_bf16(acc[f][j][0]) | ((unsigned)f32_to_bf16(acc[f][j][1]) << 16);
+        v.y = (unsigned)f32_to_bf16(acc[f][j][2]) | ((unsigned)f32_to_bf16(acc[f][j][3]) << 16);
+        const int chunk = col >> 3;  // 8 bf16 per 16-byte chunk
+        *(uint2*)(tile + xr * 512 + ((chunk ^ (xr & 7)) << 4) + (col & 7) * 2) = v;
+      }
+    }
+    __syncthreads();
+    bf16_t* y = (bf16_t*)out;
+    const int c32 = tid & 31, r16 = tid >> 5;          // 16 rows per pass
+    const int ncols = min(256, N - wrow0);
+#pragma unroll
+    for (int i = 0; i < BM / 16; ++i) {
+      const int r = r16 + 16 * i;
+      if (r < item.row_count && c32 * 8 < ncols) {
+        v4i v = *(const v4i*)(tile + r * 512 + ((c32 ^ (r & 7)) << 4));
+        *(v4i*)(y + (size_t)(item.row_start + r) * N + wrow0 + c32 * 8) = v;
+      }
+    }
+  }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(NT, 1) void grouped_gemm_classes_kernel(
+    const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
+    const uint8_t* __restrict__ w0, const float* __restrict__ sw0, const uint8_t* __restrict__ w1,
+    const float* __restrict__ sw1, const TileHeader* __restrict__ hdr, const TileEntry* __restrict__ tiles, int K,
+    int N, void* __restrict__ out, float* __restrict__ out_scale) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+  // work items = (row tile, column block) pairs in [expert][column block][row tile] order, dealt to the 8 XCDs in
+  // contiguous ranges (workgroup ids are issued round-robin over XCDs)
+  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
+  const int n_items = hdr->n_tiles * ncb;
+  const int per_xcd = (n_items + 7) >> 3;
+  const int slot = blockIdx.x >> 3;
+  const int item_id = (blockIdx.x & 7) * per_xcd + slot;
+  if (slot >= per_xcd || item_id >= n_items) return;
+  Item item;
+  {
+    const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
+    const int nt = moe_tile_count(te.rows, 256);
+    const int local = item_id - te.first_tile * ncb;
+    item.col_block = nt == 1 ? local : local / nt;
+    const int rt = local - item.col_block * nt;
+    item.expert = te.expert;
+    int t0, tn;
+    moe_tile_span(te.rows, 256, nt, rt, t0, tn);
+    item.row_start = te.row_start + t0;
+    item.row_count = tn;
+  }
+  const int rows = __builtin_amdgcn_readfirstlane(item.row_count);
+#define MOE_ITEM(XF) item_body<MODE, XF>(item, lds, xq, sx, row_ids, w0, sw0, w1, sw1, K, N, out, out_scale)
+#ifdef MOE_ONLY_XF
+  (void)rows;
+  MOE_ITEM(MOE_ONLY_XF);
+#else
+  switch ((rows + 31) >> 5) {
+    case 8: MOE_ITEM(8); break;
+    case 7: MOE_ITEM(7); break;
+    case 6: MOE_ITEM(6); break;
+    case 5: MOE_ITEM(5); break;
+    case 4: MOE_ITEM(4); break;
+    case 3: MOE_ITEM(3); break;
+    case 2: MOE_ITEM(2); break;
+    default: MOE_ITEM(1); break;
+  }
+#endif
+#undef MOE_ITEM
+}
+
 int col_blocks(int mode, int N) { return mode == MODE_GATEUP ? N / 128 : (N + 255) / 256; }
 
 int max_tiles_for(int R, int E, int bm) { return (int)((long long)(R + bm - 1) / bm + (E < R ? E : R)); }
@@ -515,22 +938,38 @@ int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const
   return moe_check_hip(hipGetLastError(), "gemm launch");
 }
 
-// MOE_GEMM_BM=32|128|256 in the environment pins the tile height for experiments; default: by shape
-int forced_xw() {
+template <int MODE>
+int launch_classes(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
+                   const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
+                   void* out, float* out_scale, void* ws, bool list_built, hipStream_t s) {
+  const TileList l = tile_list(ws, R, E, 256);
+  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, 256, l);
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_classes_kernel<MODE>, CLS_LDS_BYTES, lds_raised)) return rc;
+  const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
+  MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
+  const int grid = (int)((max_items + 7) / 8) * 8;
+  hipLaunchKernelGGL((grouped_gemm_classes_kernel<MODE>), dim3(grid), dim3(NT), CLS_LDS_BYTES, s, xq, sx, row_ids, w0,
+                     sw0, w1, sw1, l.hdr, l.tiles, K, N, out, out_scale);
+  return moe_check_hip(hipGetLastError(), "gemm launch");
+}
+
+// MOE_GEMM_BM=32|256 in the environment pins the kernel for experiments; default: by shape
+int forced_cfg() {
   static int v = [] {
     const char* e = getenv("MOE_GEMM_BM");
     return e ? atoi(e) : 0;
   }();
-  return v == 32 ? 0 : v == 128 ? 1 : v == 256 ? 2 : -1;
+  return v == 32 ? 0 : v == 256 ? 2 : -1;
 }
 
-// 256-row tiles once the average expert has more than 128 rows, 32-row tiles (two workgroups per CU: one streams
-// weights while the other starts or finishes an item) when it has at most 16, 128-row tiles between
+// Batches of at most 16 rows per expert on average run the 32-row kernel with two workgroups per CU (one streams
+// weights while the other starts or finishes an item); everything else runs the tile-class kernel.
 int tile_config(int R, int E) {
-  if (forced_xw() >= 0) return forced_xw();
-  return (long long)R > 128ll * E ? 2 : (long long)R <= 16ll * E ? 0 : 1;
+  if (forced_cfg() >= 0) return forced_cfg();
+  return (long long)R <= 16ll * E ? 0 : 2;
 }
-int tile_height(int cfg) { return cfg == 0 ? 32 : 128 * cfg; }
+int tile_height(int cfg) { return cfg == 0 ? 32 : 256; }
 
 template <int MODE>
 int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
@@ -542,15 +981,11 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
   MOE_REQUIRE((long long)N * K <= (1ll << 32) && (long long)R * K <= (1ll << 32), MOE_ERR_BAD_SHAPE,
               "gemm: one expert matrix and the activation array must each stay within 4 GB (N=%d K=%d R=%d)", N, K, R);
   if (R == 0) return MOE_OK;
-  const int cfg = tile_config(R, E);
-  if (cfg == 2)
-    return launch_cfg<MODE, 2>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
-                               list_built, s);
-  if (cfg == 0)
+  if (tile_config(R, E) == 0)
     return launch_cfg<MODE, 0>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
                                list_built, s);
-  return launch_cfg<MODE, 1>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
-                             list_built, s);
+  return launch_classes<MODE>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
+                              list_built, s);
 }
 
 }  // namespace
@@ -558,7 +993,7 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
 extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
   (void)N_out;   // the tile list does not depend on the number of output columns
   const int bm = tile_height(tile_config(R, E));
-  return sizeof(TileHeader) + (size_t)max_tiles_for(R, E, bm < 128 ? bm : 128) * sizeof(TileEntry) + 256;
+  return sizeof(TileHeader) + (size_t)max_tiles_for(R, E, bm) * sizeof(TileEntry) + 256;
 }
 
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
