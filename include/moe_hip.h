@@ -94,6 +94,20 @@ MOE_API int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const
                                uint8_t* hq, float* sh, void* ws, size_t ws_bytes,
                                moe_stream_t stream);
 
+/* The same gate/up GEMM for callers that cannot allocate device memory or carry a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.
+ * The list of row tiles that the kernels read lives in a static device array of MOE_STATIC_SCRATCH_BYTES inside
+ * the library (one copy per GPU, held until the process ends); the call allocates nothing and fails with
+ * MOE_ERR_WORKSPACE_TOO_SMALL when moe_gemm_workspace_bytes(R, E, I) exceeds that size.  All calls on one GPU
+ * share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls on one stream
+ * are ordered and safe.  Results are identical to moe_gemm_gateup_swiglu_fp8. */
+#define MOE_STATIC_SCRATCH_BYTES (1u << 20)
+MOE_API int moe_gemm_gateup_swiglu_fp8_static(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+                                      const uint8_t* w_gate, const float* sw_gate,
+                                      const uint8_t* w_up, const float* sw_up,
+                                      const int32_t* group_offsets, int E, int R, int D, int I,
+                                      uint8_t* hq, float* sh, moe_stream_t stream);
+
 /* moe.py:87 (the third ragged_dot): y = h . Wdown[e]^T, bf16 out (R, D). */
 MOE_API int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
                       const float* sw_down, const int32_t* group_offsets, int E, int R, int I,

@@ -46,7 +46,13 @@
 
 #include <type_traits>
 
+#include <mutex>
+
 #include "moe_common.h"
+
+// Tile list of moe_gemm_gateup_swiglu_fp8_static: one copy per GPU, held until the process ends.  In host code this
+// name is only a handle for hipGetSymbolAddress; kernels get the address that call returns.
+static __device__ __align__(256) unsigned char scratch[MOE_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -1017,6 +1023,43 @@ extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, co
                                           moe_stream_t stream) {
   return moe_gemm_gateup_impl(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
                               ws_bytes, false, stream);
+}
+
+namespace {
+// The device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void** out) {
+  static std::mutex mu;
+  static void* ptrs[64] = {};
+  int dev = 0;
+  if (int rc = moe_check_hip(hipGetDevice(&dev), "static scratch: hipGetDevice")) return rc;
+  MOE_REQUIRE(dev >= 0 && dev < 64, MOE_ERR_HIP, "static scratch: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    if (int rc = moe_check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "static scratch: hipGetSymbolAddress")) return rc;
+    MOE_REQUIRE(p != nullptr, MOE_ERR_HIP, "static scratch: no device address");
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return MOE_OK;
+}
+}  // namespace
+
+extern "C" int moe_gemm_gateup_swiglu_fp8_static(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+                                                 const uint8_t* w_gate, const float* sw_gate, const uint8_t* w_up,
+                                                 const float* sw_up, const int32_t* group_offsets, int E, int R,
+                                                 int D, int I, uint8_t* hq, float* sh, moe_stream_t stream) {
+  MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0, MOE_ERR_BAD_SHAPE, "gemm_gateup_static: need 1 <= E <= 1024, got E=%d R=%d", E, R);
+  const size_t need = moe_gemm_workspace_bytes(R, E, I);
+  MOE_REQUIRE(need <= (size_t)MOE_STATIC_SCRATCH_BYTES, MOE_ERR_WORKSPACE_TOO_SMALL,
+              "gemm_gateup_static: the tile list of R=%d rows, E=%d experts needs %zu bytes, the static scratch holds %u",
+              R, E, need, (unsigned)MOE_STATIC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  // the tile list (header and every entry the GEMM reads) is rewritten by this call's first kernel: nothing of
+  // an earlier call's contents is read
+  return moe_gemm_gateup_impl(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
+                              MOE_STATIC_SCRATCH_BYTES, false, stream);
 }
 
 int moe_gemm_down_impl(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
