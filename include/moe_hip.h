@@ -164,11 +164,16 @@ typedef struct MoeForwardArgs {
   int32_t* out_inv_perm;         /* (R) */
   uint8_t* out_hq;               /* (R, I) e4m3 codes of the SwiGLU output, rows in sorted order */
   float* out_sh;                 /* (R, I/128) their 1x128 scales */
+  uint8_t* out_hsq;              /* (M, SI) the same for the shared expert (needs SI > 0) */
+  float* out_shs;                /* (M, SI/128) */
+  void* out_y;                   /* (R, D) bf16 rows of the down GEMM, sorted order (what the combine gathers) */
+  void* out_ys;                  /* (M, D) bf16 rows of the shared expert's down GEMM (needs SI > 0) */
   /* router in front of the path (NULL = the caller supplies logits) */
   const void* w_router;          /* (E, D) bf16: logits = bf16(x . w_router^T), moe.py:50 */
   const void* w_shared_gate;     /* (1, D) bf16 or NULL: shared expert's output is scaled by
                                     sigmoid(x . w_shared_gate^T), moe.py:278-279; needs w_router and SI > 0 */
   float* out_logits;             /* (M, E) optional copy of the logits the router computed (else never stored) */
+  float* out_shared_gate;        /* (M) optional copy of the shared expert's gate values (needs w_shared_gate) */
   /* the steps either side of the layer (block.py:54-58, :88-91); NULL / 0 = off */
   const float* norm_weight;      /* (D) f32: x is RMS-normalised first (rms_norm with 1 + weight, in bf16) */
   float norm_eps;

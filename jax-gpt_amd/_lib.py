@@ -33,8 +33,9 @@ class MoeForwardArgs(C.Structure):
         ("out", C.c_void_p),
         ("out_idx", C.c_void_p), ("out_w", C.c_void_p), ("out_group_sizes", C.c_void_p),
         ("out_sorted_token_ids", C.c_void_p), ("out_inv_perm", C.c_void_p),
-        ("out_hq", C.c_void_p), ("out_sh", C.c_void_p),
-        ("w_router", C.c_void_p), ("w_shared_gate", C.c_void_p), ("out_logits", C.c_void_p),
+        ("out_hq", C.c_void_p), ("out_sh", C.c_void_p), ("out_hsq", C.c_void_p), ("out_shs", C.c_void_p),
+        ("out_y", C.c_void_p), ("out_ys", C.c_void_p),
+        ("w_router", C.c_void_p), ("w_shared_gate", C.c_void_p), ("out_logits", C.c_void_p), ("out_shared_gate", C.c_void_p),
         ("norm_weight", C.c_void_p), ("norm_eps", C.c_float), ("add_residual", C.c_int),
     ]
 

@@ -24,7 +24,7 @@ int moe_check_hip(hipError_t e, const char* what) {
   return moe_set_error(MOE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-extern "C" int moe_abi_version(void) { return 3; }
+extern "C" int moe_abi_version(void) { return 5; }
 extern "C" const char* moe_last_error(void) { return g_err; }
 
 namespace {
@@ -139,6 +139,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   MOE_REQUIRE(!a->w_shared_gate || (a->w_router && a->SI), MOE_ERR_NULL,
               "forward: w_shared_gate needs w_router and a shared expert");
   MOE_REQUIRE(a->w_router || !a->out_logits, MOE_ERR_NULL, "forward: out_logits is an output of the router (w_router)");
+  MOE_REQUIRE(a->w_shared_gate || !a->out_shared_gate, MOE_ERR_NULL, "forward: out_shared_gate needs w_shared_gate");
   ForwardBuffers b = carve(ws, a->M, a->D, a->E, a->k, a->I, a->SI, true);
   int32_t* idx = a->out_idx ? a->out_idx : b.idx;
   float* w = a->out_w ? a->out_w : b.w;
@@ -150,6 +151,15 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   MOE_REQUIRE(MOE_ALIGNED16(a->out_hq), MOE_ERR_BAD_ALIGN, "forward: out_hq must be 16-byte aligned");
   uint8_t* hq = a->out_hq ? a->out_hq : b.hq;
   float* sh = a->out_sh ? a->out_sh : b.sh;
+  MOE_REQUIRE((a->out_hsq == nullptr) == (a->out_shs == nullptr) && (!a->out_hsq || a->SI), MOE_ERR_NULL,
+              "forward: out_hsq and out_shs come together and need a shared expert");
+  MOE_REQUIRE(MOE_ALIGNED16(a->out_hsq), MOE_ERR_BAD_ALIGN, "forward: out_hsq must be 16-byte aligned");
+  uint8_t* hsq = a->out_hsq ? a->out_hsq : b.hsq;
+  float* shs = a->out_shs ? a->out_shs : b.shs;
+  MOE_REQUIRE(!a->out_ys || a->SI, MOE_ERR_NULL, "forward: out_ys needs a shared expert");
+  MOE_REQUIRE(MOE_ALIGNED16(a->out_y) && MOE_ALIGNED16(a->out_ys), MOE_ERR_BAD_ALIGN, "forward: out_y / out_ys must be 16-byte aligned");
+  void* y = a->out_y ? a->out_y : b.y;
+  void* ys = a->out_ys ? a->out_ys : b.ys;
   const int R = a->M * a->k;
   hipStream_t main_s = (hipStream_t)stream;
   MOE_REQUIRE(a->routing == MOE_ROUTING_SOFTMAX || a->routing == MOE_ROUTING_SIGMOID_GROUPED, MOE_ERR_BAD_SHAPE,
@@ -183,10 +193,10 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
     if (!rc_shared)
       rc_shared = moe_gemm_gateup_impl(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up, b.dense_off, 1,
-                                       a->M, a->D, a->SI, b.hsq, b.shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, false,
+                                       a->M, a->D, a->SI, hsq, shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, false,
                                        (moe_stream_t)side);
     if (!rc_shared)   // same rows, same tile height: the list the gate/up launch built serves the down launch too
-      rc_shared = moe_gemm_down_impl(b.hsq, b.shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, b.ys,
+      rc_shared = moe_gemm_down_impl(hsq, shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, ys,
                                      b.gemm_ws_shared, b.gemm_ws_shared_bytes, true, (moe_stream_t)side);
   } else {
     if ((rc = quantise(a, b, stream))) return rc;
@@ -226,8 +236,9 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     if ((rc = moe_router_partials(a->norm_weight ? b.normed : a->x, a->M, a->D, a->w_router, a->E, a->w_shared_gate,
                                   b.router_ws, b.router_ws_bytes, &splits, &n_cols, stream)))
       return join(rc);
-    if (a->w_shared_gate) shared_gate = b.shared_gate;
-    src = LogitSource{nullptr, (const float*)b.router_ws, splits, n_cols, a->out_logits, b.shared_gate};
+    float* gate_out = a->out_shared_gate ? a->out_shared_gate : b.shared_gate;   // (written by the routing kernel)
+    if (a->w_shared_gate) shared_gate = gate_out;
+    src = LogitSource{nullptr, (const float*)b.router_ws, splits, n_cols, a->out_logits, gate_out};
   }
   if (a->routing == MOE_ROUTING_SOFTMAX)
     rc = moe_route_softmax_impl(src, a->M, a->E, a->k, a->renorm, idx, w, stream);
@@ -249,10 +260,10 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   if ((rc = moe_gemm_gateup_impl(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets, a->E, R,
                                  a->D, a->I, hq, sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);
-  if ((rc = moe_gemm_down_impl(hq, sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, b.y,
+  if ((rc = moe_gemm_down_impl(hq, sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, y,
                                b.gemm_ws, b.gemm_ws_bytes, true, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;
-  return moe_combine(b.y, w, inv, a->SI ? b.ys : nullptr, shared_gate, a->add_residual ? a->x : nullptr, a->M, a->k,
+  return moe_combine(y, w, inv, a->SI ? ys : nullptr, shared_gate, a->add_residual ? a->x : nullptr, a->M, a->k,
                      a->D, a->out, stream);
 }

@@ -360,7 +360,8 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     expert's output by its sigmoid gate (moe.py:278-279).  `norm_weight` (D,) puts the
     block's RMSNorm in front (block.py:54) and `add_residual` its `x + moe_out` behind (:58).
     Returns (M, D) bf16, plus, if return_debug, a dict of the integer intermediates and of the quantised
-    SwiGLU output the down GEMM consumed (`hq` (R, I) e4m3 codes as uint8 and `sh` (R, I/128), sorted order)."""
+    SwiGLU output the down GEMMs consumed (`hq` (R, I) e4m3 codes as uint8 and `sh` (R, I/128), sorted order;
+    `hsq` (M, SI) and `shs` for the shared expert) and of the down GEMMs' rows (`y` (R, D), `ys` (M, D))."""
     x = _dev(x, torch.bfloat16, "x")
     wr = wsg = None
     if gate_weight is not None:
@@ -437,9 +438,19 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
                    inv_perm=_empty((R,), torch.int32, x),
                    hq=_empty((R, I), torch.uint8, x), sh=_empty((R, I // 128), torch.float32, x))
         a.out_hq, a.out_sh = dbg["hq"].data_ptr(), dbg["sh"].data_ptr()
+        dbg["y"] = _empty((R, D), torch.bfloat16, x)
+        a.out_y = dbg["y"].data_ptr()
+        if SI:
+            dbg["hsq"], dbg["shs"] = _empty((M, SI), torch.uint8, x), _empty((M, SI // 128), torch.float32, x)
+            a.out_hsq, a.out_shs = dbg["hsq"].data_ptr(), dbg["shs"].data_ptr()
+            dbg["ys"] = _empty((M, D), torch.bfloat16, x)
+            a.out_ys = dbg["ys"].data_ptr()
         if wr is not None:
             dbg["logits"] = _empty((M, E), torch.float32, x)
             a.out_logits = dbg["logits"].data_ptr()
+            if wsg is not None:
+                dbg["shared_gate"] = _empty((M,), torch.float32, x)
+                a.out_shared_gate = dbg["shared_gate"].data_ptr()
         a.out_idx, a.out_w = dbg["indices"].data_ptr(), dbg["weights"].data_ptr()
         a.out_group_sizes = dbg["group_sizes"].data_ptr()
         a.out_sorted_token_ids, a.out_inv_perm = dbg["sorted_token_ids"].data_ptr(), dbg["inv_perm"].data_ptr()

@@ -326,15 +326,20 @@ def silu(x):
     return x / (1.0 + np.exp(-x))
 
 
-def expert_swiglu(xq, sx, experts, group_offsets, dtype=np.float64):
+def expert_swiglu(xq, sx, experts, group_offsets, dtype=np.float64, h=None):
     """gate/up grouped GEMM -> silu(g)*u in f32 -> 1x128 fp8 quant -> down grouped GEMM.
 
     `experts` = dict(gate=(codes, scale_inv), up=..., down=...).  Returns
-    (y f32 (R,D), hq, sh) where y is rounded once to bf16-representable f32."""
-    g = grouped_gemm(xq, sx, *experts["gate"], group_offsets, dtype=dtype)
-    u = grouped_gemm(xq, sx, *experts["up"], group_offsets, dtype=dtype)
-    h = (silu(g) * u).astype(np.float32)
-    hq, sh = quant_act_group(h)
+    (y f32 (R,D), hq, sh) where y is rounded once to bf16-representable f32.
+    `h` = (codes, scale_inv) takes the place of the quantised intermediate: the second half of the path alone,
+    continued from an intermediate computed elsewhere (the tests pass the kernel's own, so that the comparison of
+    the outputs is not blurred by intermediate values that sit on an fp8 rounding boundary)."""
+    if h is None:
+        g = grouped_gemm(xq, sx, *experts["gate"], group_offsets, dtype=dtype)
+        u = grouped_gemm(xq, sx, *experts["up"], group_offsets, dtype=dtype)
+        hq, sh = quant_act_group((silu(g) * u).astype(np.float32))
+    else:
+        hq, sh = np.asarray(h[0], np.uint8), np.asarray(h[1], np.float32)
     y = grouped_gemm(hq, sh, *experts["down"], group_offsets, dtype=dtype)
     return bf16_round(y.astype(np.float32)), hq, sh
 
@@ -389,15 +394,15 @@ def shared_gate(x, shared_expert_gate_weight):
     return bf16_round(sigmoid_det(z))
 
 
-def moe_sublayer(x, moe_norm_weight, params, top_k, eps=1e-6, dtype=np.float64):
+def moe_sublayer(x, moe_norm_weight, params, top_k, eps=1e-6, dtype=np.float64, routed_h=None, shared_h=None):
     """block.py:54-58: x + moe_layer(rms_norm(x, moe_norm), params) on (M, D) rows."""
     normed = rms_norm(x, moe_norm_weight, eps)
-    r = moe_layer(normed, params, top_k, dtype=dtype, residual=x)
+    r = moe_layer(normed, params, top_k, dtype=dtype, residual=x, routed_h=routed_h, shared_h=shared_h)
     r["normed"] = normed
     return r
 
 
-def moe_layer(x, params, top_k, dtype=np.float64, residual=None):
+def moe_layer(x, params, top_k, dtype=np.float64, residual=None, routed_h=None, shared_h=None):
     """moe.py:235-282 on (M, D) rows: softmax routing on the router's own logits, routed experts,
     shared expert scaled by its sigmoid gate, one add.  params: gate_weight (D, E); experts / shared
     dicts as in moe_experts; shared_expert_gate_weight (D, 1) or absent."""
@@ -405,7 +410,7 @@ def moe_layer(x, params, top_k, dtype=np.float64, residual=None):
     r = moe_experts(x, logits, params["experts"], top_k=top_k, routing="softmax", shared=params.get("shared"),
                     shared_gate_values=(shared_gate(x, params["shared_expert_gate_weight"])
                                         if params.get("shared_expert_gate_weight") is not None else None),
-                    residual=residual, dtype=dtype)
+                    residual=residual, dtype=dtype, routed_h=routed_h, shared_h=shared_h)
     r["logits"] = logits
     return r
 
@@ -416,9 +421,11 @@ def moe_layer(x, params, top_k, dtype=np.float64, residual=None):
 
 def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=None, n_group=1,
                 topk_group=1, renorm=True, routed_scale=1.0, shared=None, shared_gate_values=None,
-                residual=None, dtype=np.float64):
+                residual=None, dtype=np.float64, routed_h=None, shared_h=None):
     """x: (M,D) float32 holding bf16-representable values.  experts/shared: dicts
-    gate/up/down -> (codes, scale_inv) with expert weights (E,N,K) and shared (1,N,K)."""
+    gate/up/down -> (codes, scale_inv) with expert weights (E,N,K) and shared (1,N,K).
+    routed_h / shared_h = (codes, scale_inv): continue from these quantised intermediates (rows in sorted
+    order / token order) instead of computing them (see expert_swiglu)."""
     E = experts["gate"][0].shape[0]
     if routing == "softmax":
         idx, w = route_softmax_topk(router_logits, top_k, renorm)
@@ -429,37 +436,53 @@ def moe_experts(x, router_logits, experts, *, top_k, routing="softmax", bias=Non
     sg = sort_and_group(idx, E)
     xq, sx = quant_act_group(x)
     xs, sxs = xq[sg["sorted_token_ids"]], sx[sg["sorted_token_ids"]]        # moe.py:79
-    y, hq, sh = expert_swiglu(xs, sxs, experts, sg["group_offsets"], dtype=dtype)
-    ys = None
+    y, hq, sh = expert_swiglu(xs, sxs, experts, sg["group_offsets"], dtype=dtype, h=routed_h)
+    ys = hsq = shs = None
     if shared is not None:
         M = x.shape[0]
-        ys, _, _ = expert_swiglu(xq, sx, shared, np.array([0, M], dtype=np.int32), dtype=dtype)
+        ys, hsq, shs = expert_swiglu(xq, sx, shared, np.array([0, M], dtype=np.int32), dtype=dtype, h=shared_h)
     out = combine(y, w, sg["inv_perm"], ys, shared_gate_values, residual)
-    return dict(out=out, indices=idx, weights=w, xq=xq, sx=sx, y=y, hq=hq, sh=sh, shared_out=ys, **sg)
+    return dict(out=out, indices=idx, weights=w, xq=xq, sx=sx, y=y, hq=hq, sh=sh, shared_out=ys, hsq=hsq, shs=shs, **sg)
 
 
 def moe_experts_rows(x, tokens, indices, weights, fetch_expert, shared=None, dtype=np.float64, shared_gate_values=None,
-                     residual=None):
+                     residual=None, routed_h=None, shared_h=None, return_h=False):
     """The same mathematics for a handful of token rows at full problem size:
     `fetch_expert(e)` returns dict gate/up/down -> (codes (N,K), scale_inv) for
     expert e.  shared_gate_values (M,) and residual (M, D) as in combine.
-    Returns (len(tokens), D) f32 (bf16-representable)."""
-    outs = []
-    for t in tokens:
+    routed_h = (codes (len(tokens), k, I), scale_inv (len(tokens), k, I/128)) and shared_h = (codes (len(tokens), SI),
+    scale_inv) continue from given intermediates (see expert_swiglu).
+    Returns (len(tokens), D) f32 (bf16-representable); with return_h a dict: out, the intermediates this function
+    computed or was given (routed_h, shared_h, in the layout of the arguments) and the bf16 rows the combine summed
+    (y (len(tokens), k, D), ys (len(tokens), D) or None)."""
+    outs, hs, hss, yrows, ysrows = [], [], [], [], []
+    for ti, t in enumerate(tokens):
         xq, sx = quant_act_group(x[t:t + 1])
         acc = np.zeros((1, x.shape[1]), dtype=np.float32)
         off = np.array([0, 1], dtype=np.int32)
+        row_h = []
         for s in range(indices.shape[1]):
             ex = fetch_expert(int(indices[t, s]))
             ex = {n: (q[None], sc[None]) for n, (q, sc) in ex.items()}
-            y, _, _ = expert_swiglu(xq, sx, ex, off, dtype=dtype)
+            hin = None if routed_h is None else (routed_h[0][ti, s][None], routed_h[1][ti, s][None])
+            y, hq1, sh1 = expert_swiglu(xq, sx, ex, off, dtype=dtype, h=hin)
+            row_h.append((hq1[0], sh1[0], y[0]))
             acc = (acc + y * np.float32(weights[t, s])).astype(np.float32)
+        hs.append(row_h)
         if shared is not None:
-            ys, _, _ = expert_swiglu(xq, sx, shared, off, dtype=dtype)
+            hin = None if shared_h is None else (shared_h[0][ti][None], shared_h[1][ti][None])
+            ys, hq1, sh1 = expert_swiglu(xq, sx, shared, off, dtype=dtype, h=hin)
+            hss.append((hq1[0], sh1[0]))
+            ysrows.append(ys[0])
             if shared_gate_values is not None:
                 ys = (ys * np.float32(shared_gate_values[t])).astype(np.float32)
             acc = (acc + ys).astype(np.float32)
         if residual is not None:
             acc = (acc + residual[t:t + 1].astype(np.float32)).astype(np.float32)
         outs.append(bf16_round(acc)[0])
-    return np.stack(outs)
+    if not return_h:
+        return np.stack(outs)
+    rh = (np.stack([np.stack([q for q, _, _ in r]) for r in hs]), np.stack([np.stack([sc for _, sc, _ in r]) for r in hs]))
+    sh_ = (np.stack([q for q, _ in hss]), np.stack([sc for _, sc in hss])) if hss else None
+    return dict(out=np.stack(outs), routed_h=rh, shared_h=sh_, y=np.stack([np.stack([yy for _, _, yy in r]) for r in hs]),
+                ys=np.stack(ysrows) if ysrows else None)

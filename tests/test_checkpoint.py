@@ -101,10 +101,17 @@ def test_qwen35_ingest_runs_the_layer():
     xn = x.reshape(-1, D).float().cpu().numpy()
     wr = sd["model.layers.3.mlp.gate.weight"].float().numpy().T
     wg = sd["model.layers.3.mlp.shared_expert_gate.weight"].float().numpy().T
-    logits = jg.router_logits(x.reshape(-1, D), pq["gate_weight"]).cpu().numpy()
-    ref = O.moe_experts(xn, logits, experts, top_k=k, shared=shared, shared_gate_values=O.shared_gate(xn, wg))
+    a2, dbg = jg.moe_experts(x.reshape(-1, D), None, top_k=k,
+                             experts={n: pq[n] for n in ("gate_proj", "up_proj", "down_proj")},
+                             shared={n: pq["shared_" + n] for n in ("gate_proj", "up_proj", "down_proj")},
+                             gate_weight=pq["gate_weight"], shared_expert_gate_weight=pq["shared_expert_gate_weight"],
+                             return_debug=True)
+    assert torch.equal(a2, a.reshape(-1, D))
+    logits = dbg["logits"].cpu().numpy()
     assert float((logits != O.router_logits(xn, wr)).mean()) < 0.01
-    H.assert_close_out(H.bf16_to_np(a.reshape(-1, D)), ref["out"], tol=1e-2, inner=I)
+    gate_k = H.kernel_gate(dbg, O.shared_gate(xn, wg))
+    oracle = lambda **h: O.moe_experts(xn, logits, experts, top_k=k, shared=shared, shared_gate_values=gate_k, **h)
+    H.check_layer_output(a2, dbg, oracle(), oracle, shared_gate=gate_k)
 
 
 @pytest.mark.gpu
@@ -125,10 +132,11 @@ def test_block_fp8_ingest_runs_the_layer():
                             shared=H.experts_to_cuda(prob["shared"]), routing="sigmoid_grouped", bias=H.to_cuda(prob["bias"]),
                             n_group=4, topk_group=2)
     assert torch.equal(out, direct)
-    ref = O.moe_experts(prob["x"], dbg["logits"].cpu().numpy(), prob["experts"], top_k=2, shared=prob["shared"],
-                        routing="sigmoid_grouped", bias=prob["bias"], n_group=4, topk_group=2)
+    oracle = lambda **h: O.moe_experts(prob["x"], dbg["logits"].cpu().numpy(), prob["experts"], top_k=2, shared=prob["shared"],
+                                       routing="sigmoid_grouped", bias=prob["bias"], n_group=4, topk_group=2, **h)
+    ref = oracle()
     assert np.array_equal(dbg["indices"].cpu().numpy(), ref["indices"])
-    H.assert_close_out(H.bf16_to_np(out), ref["out"], tol=1e-2, inner=128)
+    H.check_layer_output(out, dbg, ref, oracle)
 
 
 def _qwen3_moe_sd(E, D, I, seed, prefix="model.layers.1"):

@@ -4,7 +4,11 @@ The oracle cannot run these sizes in full, so each test checks
   * every integer result (routing indices, group sizes, permutation) exactly against
     the oracle, which is cheap at any size;
   * the bf16 output on a sample of token rows against the oracle's per-row path
-    (weights of the sampled tokens' experts are copied back from the GPU);
+    (weights of the sampled tokens' experts are copied back from the GPU), split at the fp8
+    intermediate h as helpers.check_layer_output does: the kernel's h rows against the oracle's,
+    and the output rows against the oracle continued from the kernel's h, to the plain
+    tolerance (1e-2 max-normalised and allclose);
+  * at config 3 every row of one expert that spans two row tiles, through the stage entry points;
   * size-independent properties: a sub-batch gives bit-identical rows; every routed
     row is written exactly once; empty experts are skipped.
 Weights are generated on the GPU (the DeepSeek-V3 shape is 11.3 GB of fp8) by the same
@@ -46,6 +50,72 @@ def _fetch(experts):
     return f
 
 
+def _check_sampled_rows(outn, x_rows, tokens, ridx, rw, experts, shared, dbg, k, shared_gate_values=None, residual=None):
+    """The sampled tokens against the oracle, stage by stage as helpers.check_layer_output does for whole layers:
+    the kernel's h rows against the oracle's; its down-GEMM rows against the oracle continued from its h; its output
+    rows bit for bit against the oracle's combine of its own rows; the output against the oracle continued from its
+    h.  One token per worker thread (NumPy releases the interpreter lock inside its big operations), float32 BLAS
+    as the oracle allows for big shapes."""
+    import torch
+    from concurrent.futures import ThreadPoolExecutor
+    fetch = _fetch(experts)
+    cache = {e: fetch(e) for e in sorted({int(e) for t in tokens for e in ridx[t]})}
+    sh = None
+    if shared is not None:
+        f = _fetch(shared)(0)
+        sh = {n: (q[None], s[None]) for n, (q, s) in f.items()}
+    n = len(tokens)
+    inv = dbg["inv_perm"].cpu().numpy().reshape(-1, k)
+    pos = torch.from_numpy(np.ascontiguousarray(inv[tokens].reshape(-1))).cuda().long()
+    khq = H.codes_np(dbg["hq"][pos]).reshape(n, k, -1)
+    ksh = dbg["sh"][pos].cpu().numpy().reshape(n, k, -1)
+    ky = H.bf16_to_np(dbg["y"][pos])                                   # (n * k, D), token-major
+    kshared = kys = None
+    if shared is not None:
+        tsel = torch.tensor(tokens, device="cuda")
+        kshared = (H.codes_np(dbg["hsq"][tsel]), dbg["shs"][tsel].cpu().numpy())
+        kys = H.bf16_to_np(dbg["ys"][tsel])
+    D = x_rows.shape[1]
+    xfull = np.zeros((max(tokens) + 1, D), np.float32)
+    xfull[tokens] = x_rows
+
+    def one(i):
+        t = tokens[i]
+        kw = dict(shared=sh, dtype=np.float32, shared_gate_values=shared_gate_values, residual=residual, return_h=True)
+        own = O.moe_experts_rows(xfull, [t], ridx, rw, cache.__getitem__, **kw)
+        cont = O.moe_experts_rows(xfull, [t], ridx, rw, cache.__getitem__, routed_h=(khq[i:i + 1], ksh[i:i + 1]),
+                                  shared_h=None if kshared is None else (kshared[0][i:i + 1], kshared[1][i:i + 1]), **kw)
+        return own, cont
+
+    with ThreadPoolExecutor(max_workers=16) as pool:
+        res = list(pool.map(one, range(n)))
+    cat = lambda which, key: np.concatenate([r[which][key] for r in res])
+    I = khq.shape[-1]
+    oh = (np.concatenate([r[0]["routed_h"][0] for r in res]), np.concatenate([r[0]["routed_h"][1] for r in res]))
+    frac = H.assert_h_close(khq.reshape(-1, I), ksh.reshape(-1, I // 128), oh[0].reshape(-1, I), oh[1].reshape(-1, I // 128),
+                            "routed h of the sampled rows")
+    if shared is not None:
+        H.assert_h_close(kshared[0], kshared[1], np.concatenate([r[0]["shared_h"][0] for r in res]),
+                         np.concatenate([r[0]["shared_h"][1] for r in res]), "shared h of the sampled rows")
+    y_ref = cat(1, "y").reshape(n * k, D)
+    H.assert_close_out(ky, y_ref, tol=1e-2)
+    ys_ref = cat(1, "ys") if shared is not None else None
+    if shared is not None:
+        H.assert_close_out(kys, ys_ref, tol=1e-2)
+    w_rows = dbg["weights"].cpu().numpy()[tokens]
+    ident = np.arange(n * k, dtype=np.int32)
+    g_rows = None if shared_gate_values is None else np.asarray(shared_gate_values)[tokens]
+    r_rows = None if residual is None else np.asarray(residual)[tokens]
+    assert np.array_equal(outn[tokens], O.combine(ky, w_rows, ident, kys, g_rows, r_rows)), \
+        "sampled output rows are not the exact combine of the kernel's own rows"
+    cont_out, own_out = cat(1, "out"), cat(0, "out")
+    err = H.max_norm_err(outn[tokens], cont_out)
+    assert err <= 1e-2, f"max-normalised error {err:.3e}"
+    leaning = H.assert_allclose_but_for_row_steps(outn[tokens], cont_out, ky, y_ref, kys, ys_ref, w_rows, ident, g_rows, 1e-2)
+    _say(f"   {n} sampled rows: max-normalised error {err:.2e} from the kernel's h ({frac:.2%} of its codes differ from "
+         f"the oracle's; {leaning} output elements lean on a row's bf16 step; end to end {H.max_norm_err(outn[tokens], own_out):.2e})")
+
+
 def _check_layer(jg, torch, cfg, layer, seed, n_sample):
     experts, shared, bias, _ = layer
     gen = torch.Generator(device="cuda")
@@ -80,21 +150,13 @@ def _check_layer(jg, torch, cfg, layer, seed, n_sample):
     rng = H.rng_for(seed)
     tokens = sorted(set([0, M - 1] + list(rng.integers(0, M, n_sample - 2))))
     xs = H.bf16_to_np(x[torch.tensor(tokens, device="cuda")])
-    xfull = np.zeros((max(tokens) + 1, D), np.float32)
-    xfull[tokens] = xs
-    sh = None
-    if shared is not None:
-        f = _fetch(shared)(0)
-        sh = {n: (q[None], s[None]) for n, (q, s) in f.items()}
-    want = O.moe_experts_rows(xfull, tokens, ridx, rw, _fetch(experts), shared=sh)
-    err = H.assert_close_out(outn[tokens], want, tol=1e-2, inner=I)
-    _say(f"   {len(tokens)} sampled rows: max-normalised error {err:.2e}")
+    _check_sampled_rows(outn, xs, tokens, ridx, rw, experts, shared, dbg, k)
 
     # a sub-batch gives the same rows, bit for bit (a row's arithmetic does not depend on its tile)
     nsub = min(M, 96)
     part = jg.moe_experts(x[:nsub].contiguous(), logits[:nsub].contiguous(), **kw)
     assert torch.equal(out[:nsub], part)
-    return out
+    return out, dbg, x
 
 
 def test_config2_qwen3_moe_prefill(env):
@@ -102,7 +164,7 @@ def test_config2_qwen3_moe_prefill(env):
     _say("config 2: Qwen3-MoE-style prefill")
     cfg = bench.WORKLOADS["qwen3_moe_prefill"]
     layer = bench.make_layer(jg, torch, cfg, seed=2)
-    _check_layer(jg, torch, cfg, layer, seed=20, n_sample=16)
+    _check_layer(jg, torch, cfg, layer, seed=20, n_sample=32)
 
 
 @pytest.fixture(scope="module")
@@ -114,13 +176,48 @@ def dsv3_layer(env):
 def test_config3_deepseek_v3_prefill(env, dsv3_layer):
     jg, torch, bench = env
     _say("config 3: DeepSeek-V3-style prefill")
-    _check_layer(jg, torch, bench.WORKLOADS["deepseek_v3_prefill"], dsv3_layer, seed=30, n_sample=4)
+    cfg = bench.WORKLOADS["deepseek_v3_prefill"]
+    out, dbg, x = _check_layer(jg, torch, cfg, dsv3_layer, seed=30, n_sample=32)
+    _check_whole_expert(jg, torch, cfg, dsv3_layer, dbg, x)
+
+
+def _check_whole_expert(jg, torch, cfg, layer, dbg, x):
+    """Every row of one expert that is cut into two row tiles (257 .. 512 rows; both tiles, their first and last
+    rows, the rows either side of the cut) through the stage entry points at K = 7168: the gate/up GEMM's h against
+    the oracle's, and the down GEMM's rows against the oracle continued from that h, to the plain tolerance."""
+    experts = layer[0]
+    E, D, I = cfg["E"], cfg["D"], cfg["I"]
+    gs = dbg["group_sizes"].cpu().numpy()
+    cand = np.nonzero((gs > 256) & (gs <= 512))[0]
+    assert cand.size, "no expert with two row tiles in this routing"
+    e = int(cand[np.argmin(np.abs(gs[cand] - 292))])
+    off = np.concatenate([[0], np.cumsum(gs)]).astype(np.int32)
+    a, b = int(off[e]), int(off[e + 1])
+    _say(f"   whole expert {e}: rows {a}..{b} ({b - a} rows, two row tiles)")
+    xq, sx = jg.quant_act(x)
+    d_off = H.to_cuda(off)
+    stid = dbg["sorted_token_ids"]
+    hq, sh = jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], d_off, row_ids=stid)
+    assert torch.equal(hq.view(torch.uint8), dbg["hq"]) and torch.equal(sh, dbg["sh"])      # the stage call = the layer call
+    y = jg.gemm_down(hq, sh, experts["down_proj"], d_off)
+    rows = stid[a:b].long()
+    xe_q, xe_s = H.codes_np(xq[rows]), sx[rows].cpu().numpy()
+    ex = {n: (q[None], s[None]) for n, (q, s) in _fetch(experts)(e).items()}
+    o1 = np.array([0, b - a], np.int32)
+    g = O.grouped_gemm(xe_q, xe_s, *ex["gate"], o1, dtype=np.float32)
+    u = O.grouped_gemm(xe_q, xe_s, *ex["up"], o1, dtype=np.float32)
+    rhq, rsh = O.quant_act_group((O.silu(g.astype(np.float64)) * u).astype(np.float32))
+    khq, ksh = H.codes_np(hq[a:b]), sh[a:b].cpu().numpy()
+    frac = H.assert_h_close(khq, ksh, rhq, rsh, "h of the whole expert")
+    want = O.bf16_round(O.grouped_gemm(khq, ksh, *ex["down"], o1, dtype=np.float32).astype(np.float32))
+    err = H.assert_close_out(H.bf16_to_np(y[a:b]), want, tol=1e-2)
+    _say(f"   whole expert: {frac:.2%} of h codes differ from the oracle's; down GEMM rows max-normalised error {err:.2e}")
 
 
 def test_config4_deepseek_v3_decode(env, dsv3_layer):
     jg, torch, bench = env
     _say("config 4: DeepSeek-V3-style decode")
-    _check_layer(jg, torch, bench.WORKLOADS["deepseek_v3_decode"], dsv3_layer, seed=40, n_sample=4)
+    _check_layer(jg, torch, bench.WORKLOADS["deepseek_v3_decode"], dsv3_layer, seed=40, n_sample=32)
 
 
 def test_config5_expert_parallel_shard_skewed(env):
@@ -160,17 +257,28 @@ def test_config5_expert_parallel_shard_skewed(env):
     fetch = _fetch(experts)
     nz = np.nonzero(group_sizes)[0]
     big, small = nz[np.argmax(group_sizes[nz])], nz[np.argmin(group_sizes[nz])]
-    rows = sorted(set([int(off[big]), int(off[big + 1] - 1), int(off[small]), int(off[small + 1] - 1)] + list(rng.integers(0, R, 4))))
-    xsn = H.bf16_to_np(xs[torch.tensor(rows, device="cuda")])
-    want = []
-    for i, r in enumerate(rows):
-        e = int(rows_expert[r])
-        ex = {n: (q[None], s[None]) for n, (q, s) in fetch(e).items()}
+    rows = sorted(set([int(off[big]), int(off[big + 1] - 1), int(off[small]), int(off[small + 1] - 1)] + list(rng.integers(0, R, 28))))
+    rsel = torch.tensor(rows, device="cuda")
+    xsn = H.bf16_to_np(xs[rsel])
+    khq, ksh = H.codes_np(hq[rsel]), sh[rsel].cpu().numpy()
+    cache = {e: fetch(e) for e in sorted({int(rows_expert[r]) for r in rows})}
+    one_row = np.array([0, 1], np.int32)
+
+    def one(i):
+        ex = {n: (q[None], s[None]) for n, (q, s) in cache[int(rows_expert[rows[i]])].items()}
         q1, s1 = O.quant_act_group(xsn[i:i + 1])
-        yy, _, _ = O.expert_swiglu(q1, s1, ex, np.array([0, 1], np.int32))
-        want.append(yy[0])
-    err = H.assert_close_out(yn[rows], np.stack(want), tol=1e-2, inner=I)
-    _say(f"   {len(rows)} sampled rows: max-normalised error {err:.2e}; group sizes min/max {group_sizes[nz].min()}/{group_sizes.max()}")
+        own, ohq, osh = O.expert_swiglu(q1, s1, ex, one_row, dtype=np.float32)
+        cont, _, _ = O.expert_swiglu(q1, s1, ex, one_row, dtype=np.float32, h=(khq[i:i + 1], ksh[i:i + 1]))
+        return own[0], cont[0], ohq[0], osh[0]
+
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=16) as pool:
+        res = list(pool.map(one, range(len(rows))))
+    frac = H.assert_h_close(khq, ksh, np.stack([r[2] for r in res]), np.stack([r[3] for r in res]), "h of the sampled rows")
+    err = H.assert_close_out(yn[rows], np.stack([r[1] for r in res]), tol=1e-2)
+    _say(f"   {len(rows)} sampled rows: max-normalised error {err:.2e} from the kernel's h ({frac:.2%} of its codes differ; "
+         f"end to end {H.max_norm_err(yn[rows], np.stack([r[0] for r in res])):.2e}); "
+         f"group sizes min/max {group_sizes[nz].min()}/{group_sizes.max()}")
     # the combine of the GPU's own y is exact arithmetic (f32 sum in slot order, one bf16 rounding)
     toks = [0, 1, M - 1] + list(rng.integers(0, M, 5))
     want_out = O.combine(yn, weights, inv_perm)[toks]
@@ -198,7 +306,7 @@ def test_config3_sized_moe_sublayer(env, dsv3_layer):
     outn = H.bf16_to_np(out)
     assert np.isfinite(outn).all()
     rng = H.rng_for(51)
-    tokens = sorted(set([0, M - 1] + list(rng.integers(0, M, 2))))
+    tokens = sorted(set([0, M - 1] + list(rng.integers(0, M, 30))))
     tsel = torch.tensor(tokens, device="cuda")
     xs = H.bf16_to_np(x[tsel])
     wrn, wgn, wnn = H.bf16_to_np(wr), H.bf16_to_np(wg), wn.cpu().numpy()
@@ -217,11 +325,9 @@ def test_config3_sized_moe_sublayer(env, dsv3_layer):
     assert np.array_equal(dbg["group_sizes"].cpu().numpy(), sg["group_sizes"])
     assert np.array_equal(dbg["inv_perm"].cpu().numpy(), sg["inv_perm"])
     # sampled output rows
-    f = _fetch(shared)(0)
-    sh = {n: (q[None], s[None]) for n, (q, s) in f.items()}
-    nfull = np.zeros((max(tokens) + 1, D), np.float32); nfull[tokens] = normed_gpu
-    xfull = np.zeros_like(nfull); xfull[tokens] = xs
-    gate = np.zeros(max(tokens) + 1, np.float32); gate[tokens] = O.shared_gate(normed_gpu, wgn)
-    want = O.moe_experts_rows(nfull, tokens, ridx, rw, _fetch(experts), shared=sh, shared_gate_values=gate, residual=xfull)
-    err = H.assert_close_out(outn[tokens], want, tol=1e-2, inner=I)
-    _say(f"   {len(tokens)} sampled rows: max-normalised error {err:.2e}")
+    xfull = np.zeros((max(tokens) + 1, D), np.float32); xfull[tokens] = xs
+    gate = np.zeros(max(tokens) + 1, np.float32); og = O.shared_gate(normed_gpu, wgn)
+    kg = dbg["shared_gate"].cpu().numpy()[tokens]
+    assert np.abs(kg - og).max() <= 2.0 ** -7 and int((kg != og).sum()) <= 2
+    gate[tokens] = kg
+    _check_sampled_rows(outn, normed_gpu, tokens, ridx, rw, experts, shared, dbg, k, shared_gate_values=gate, residual=xfull)

@@ -1,6 +1,9 @@
 """Parity of the HIP path (through the C ABI) against the CPU oracle on identical
-seeded inputs.  Integer results must match exactly; bf16 outputs within
-max|y-ref|/max|ref| <= 1e-2 and allclose(rtol=1e-2, atol=1e-2*rms(ref))."""
+seeded inputs.  Integer results must match exactly.  bf16 outputs must satisfy
+max|y-ref|/max|ref| <= 1e-2 and allclose(rtol=1e-2, atol=1e-2*rms(ref)); for the whole
+path the comparison is split at the fp8 intermediate h (helpers.check_layer_output): the
+kernel's h against the oracle's (codes equal but for <0.5 % that sit on a rounding
+boundary, one step apart), and the output against the oracle continued from the kernel's h."""
 import numpy as np
 import pytest
 
@@ -216,12 +219,15 @@ def _run_full(jg, prob, top_k, **kw):
     bias = None if prob["bias"] is None else H.to_cuda(prob["bias"])
     out, dbg = jg.moe_experts(H.to_bf16_cuda(prob["x"]), H.to_cuda(prob["logits"]), top_k=top_k, experts=ex, shared=sh,
                               bias=bias, return_debug=True, **kw)
-    ref = O.moe_experts(prob["x"], prob["logits"], prob["experts"], top_k=top_k, shared=prob["shared"], bias=prob["bias"], **kw)
+    oracle = lambda **h: O.moe_experts(prob["x"], prob["logits"], prob["experts"], top_k=top_k, shared=prob["shared"],
+                                       bias=prob["bias"], **kw, **h)
+    ref = oracle()
     for name in ("indices", "group_sizes", "sorted_token_ids", "inv_perm"):
         assert np.array_equal(dbg[name].cpu().numpy(), ref[name]), name
     assert np.allclose(dbg["weights"].cpu().numpy(), ref["weights"], rtol=2e-6, atol=1e-9)
-    err = H.assert_close_out(H.bf16_to_np(out), ref["out"], tol=1e-2, inner=prob["experts"]["down"][0].shape[2])
-    _say("   max-normalised error", err)
+    err, loose, frac = H.check_layer_output(out, dbg, ref, oracle)
+    _say(f"   max-normalised error {err:.2e} from the kernel's h ({frac:.2%} of its codes differ from the oracle's; "
+         f"end to end {loose:.2e})")
     return out, ref
 
 
@@ -272,9 +278,22 @@ def test_reference_entry_points(jg):
     routed = jg.expert_forward_single(x, idx, w, ex["gate_proj"], ex["up_proj"], ex["down_proj"])
     shared = jg.shared_expert_forward(x, sh["gate_proj"], sh["up_proj"], sh["down_proj"])
     ref = O.moe_experts(prob["x"], prob["logits"], prob["experts"], top_k=2, shared=prob["shared"])
-    ref_routed = O.combine(ref["y"], ref["weights"], ref["inv_perm"])
-    H.assert_close_out(H.bf16_to_np(routed), ref_routed, inner=256)
-    H.assert_close_out(H.bf16_to_np(shared), ref["shared_out"], inner=128)
+    # the same kernels called one by one expose the intermediate h: the outputs are held to the tolerance against
+    # the oracle continued from it
+    import torch
+    sg = jg.permute(idx, 8)
+    xq, sx = jg.quant_act(x)
+    hq, shh = jg.gemm_gateup_swiglu(xq, sx, ex["gate_proj"], ex["up_proj"], sg["group_offsets"], row_ids=sg["sorted_token_ids"])
+    off1 = torch.tensor([0, 96], dtype=torch.int32, device="cuda")
+    hsq, shs = jg.gemm_gateup_swiglu(xq, sx, sh["gate_proj"], sh["up_proj"], off1)
+    H.assert_h_close(H.codes_np(hq), shh.cpu().numpy(), ref["hq"], ref["sh"], "routed h")
+    H.assert_h_close(H.codes_np(hsq), shs.cpu().numpy(), ref["hsq"], ref["shs"], "shared h")
+    assert torch.equal(routed, jg.combine(jg.gemm_down(hq, shh, ex["down_proj"], sg["group_offsets"]), w, sg["inv_perm"]))
+    assert torch.equal(shared, jg.gemm_down(hsq, shs, sh["down_proj"], off1))
+    ref2 = O.moe_experts(prob["x"], prob["logits"], prob["experts"], top_k=2, shared=prob["shared"],
+                         routed_h=(H.codes_np(hq), shh.cpu().numpy()), shared_h=(H.codes_np(hsq), shs.cpu().numpy()))
+    H.assert_close_out(H.bf16_to_np(routed), O.combine(ref2["y"], ref2["weights"], ref2["inv_perm"]))
+    H.assert_close_out(H.bf16_to_np(shared), ref2["shared_out"])
 
 
 def test_graph_replay_matches_eager(jg):
@@ -398,12 +417,14 @@ def test_moe_layer_full_parity(jg):
     assert torch.equal(out.reshape(B * T, D), out2)
     logits = dbg["logits"].cpu().numpy()
     _check_logits(logits, O.router_logits(prob["x"], wr), np.abs(prob["x"]).astype(np.float64) @ np.abs(wr).astype(np.float64))
-    ref = O.moe_experts(prob["x"], logits, prob["experts"], top_k=k, shared=prob["shared"],
-                        shared_gate_values=O.shared_gate(prob["x"], wg))
+    gate_k = H.kernel_gate(dbg, O.shared_gate(prob["x"], wg))
+    oracle = lambda **h: O.moe_experts(prob["x"], logits, prob["experts"], top_k=k, shared=prob["shared"],
+                                       shared_gate_values=gate_k, **h)
+    ref = oracle()
     for name in ("indices", "group_sizes", "sorted_token_ids", "inv_perm"):
         assert np.array_equal(dbg[name].cpu().numpy(), ref[name]), name
-    err = H.assert_close_out(H.bf16_to_np(out2), ref["out"], tol=1e-2, inner=I)
-    _say("   max-normalised error", err)
+    err, loose, _ = H.check_layer_output(out2, dbg, ref, oracle, shared_gate=gate_k)
+    _say(f"   max-normalised error {err:.2e} (end to end {loose:.2e})")
     # the gate matters: without it the output differs
     no_gate = jg.moe_experts(x3.reshape(B * T, D), None, top_k=k, experts=ex, shared=sh, gate_weight=params["gate_weight"])
     assert not torch.equal(no_gate, out2)
@@ -489,12 +510,14 @@ def test_moe_sublayer_full_parity(jg):
     assert float((normed != want_n).mean()) < 0.01
     logits = dbg["logits"].cpu().numpy()
     _check_logits(logits, O.router_logits(normed, wr), np.abs(normed).astype(np.float64) @ np.abs(wr).astype(np.float64))
-    ref = O.moe_experts(normed, logits, prob["experts"], top_k=k, shared=prob["shared"],
-                        shared_gate_values=O.shared_gate(normed, wg), residual=x)
+    gate_k = H.kernel_gate(dbg, O.shared_gate(normed, wg))
+    oracle = lambda **h: O.moe_experts(normed, logits, prob["experts"], top_k=k, shared=prob["shared"],
+                                       shared_gate_values=gate_k, residual=x, **h)
+    ref = oracle()
     for name in ("indices", "group_sizes", "sorted_token_ids", "inv_perm"):
         assert np.array_equal(dbg[name].cpu().numpy(), ref[name]), name
-    err = H.assert_close_out(H.bf16_to_np(out2), ref["out"], tol=1e-2, inner=I)
-    _say("   max-normalised error", err)
+    err, loose, _ = H.check_layer_output(out2, dbg, ref, oracle, shared_gate=gate_k, residual=x)
+    _say(f"   max-normalised error {err:.2e} (end to end {loose:.2e})")
     # the unfused composition gives the same bits: norm, then the layer, then the residual added in the combine
     layer = jg.moe_experts(torch.from_numpy(normed).to(torch.bfloat16).cuda(), None, top_k=k, experts=ex, shared=sh,
                            gate_weight=params["gate_weight"], shared_expert_gate_weight=params["shared_expert_gate_weight"])
@@ -627,7 +650,7 @@ def test_concurrent_calls_on_two_streams(jg):
 @pytest.mark.parametrize("seed", [11, 12, 13])
 def test_random_shapes_full_parity(jg, seed):
     """Twelve random small layers per seed, both routers, with and without a shared expert (any intermediate size),
-    renormalised or not: integers bit-exact, outputs within the tolerance of helpers.assert_close_out."""
+    renormalised or not: integers bit-exact, outputs held to helpers.check_layer_output."""
     rng = np.random.default_rng(seed)
     for it in range(12):
         D = int(rng.integers(1, 9)) * 128
@@ -674,11 +697,13 @@ def test_moe_layer_random_shapes(jg, seed):
                                   shared_expert_gate_weight=H.to_bf16_cuda(wg) if gate else None, return_debug=True)
         logits = dbg["logits"].cpu().numpy()
         _check_logits(logits, O.router_logits(prob["x"], wr), np.abs(prob["x"]).astype(np.float64) @ np.abs(wr).astype(np.float64))
-        ref = O.moe_experts(prob["x"], logits, prob["experts"], top_k=k, shared=prob["shared"],
-                            shared_gate_values=O.shared_gate(prob["x"], wg) if gate else None)
+        gate_k = H.kernel_gate(dbg, O.shared_gate(prob["x"], wg)) if gate else None
+        oracle = lambda **h: O.moe_experts(prob["x"], logits, prob["experts"], top_k=k, shared=prob["shared"],
+                                           shared_gate_values=gate_k, **h)
+        ref = oracle()
         for name in ("indices", "group_sizes", "sorted_token_ids", "inv_perm"):
             assert np.array_equal(dbg[name].cpu().numpy(), ref[name]), name
-        H.assert_close_out(H.bf16_to_np(out), ref["out"], tol=1e-2, inner=I)
+        H.check_layer_output(out, dbg, ref, oracle, shared_gate=gate_k)
         # the stand-alone router entry point gives the same logits as the fused finish inside the layer call
         lg2 = jg.router_logits(H.to_bf16_cuda(prob["x"]), H.to_bf16_cuda(wr))
         lg2 = lg2[0] if isinstance(lg2, tuple) else lg2

@@ -315,8 +315,9 @@ def test_combine_expert_relabel_invariance_and_special_cases():
     inv = np.argsort(perm)
     lg2 = logits[:, perm]
     res2 = O.moe_experts(x, lg2, ex2, top_k=2)
-    assert np.array_equal(inv[base["indices"]], res2["indices"]) or True
-    assert np.allclose(base["out"], res2["out"], rtol=1e-2, atol=1e-6)
+    assert np.array_equal(inv[base["indices"]], res2["indices"])      # the same experts under their new names, same order
+    assert np.allclose(base["weights"], res2["weights"], rtol=1e-6, atol=0)   # (the softmax sums E terms in another order)
+    assert np.allclose(base["out"], res2["out"], rtol=2.0 ** -7, atol=1e-6)   # at most one bf16 step apart
     # k = 1 with weight 1: output is exactly the selected expert's bf16 row
     r1 = O.moe_experts(x, logits, experts, top_k=1)
     assert np.allclose(r1["weights"], 1.0)
@@ -428,3 +429,27 @@ def test_combine_residual():
     got = O.combine(y, w, inv, residual=res)
     want = np.stack([sum(np.float64(w[t, s]) * y[inv[t * k + s]] for s in range(k)) + res[t] for t in range(M)])
     assert np.abs(got - want).max() < 0.03
+
+
+def test_continuing_from_given_intermediates_reproduces_the_path():
+    """The h overrides (expert_swiglu / moe_experts / moe_experts_rows) are the second half of the same path: fed
+    the path's own intermediates they give its own output, fed other codes they give another one."""
+    x, logits, experts, shared = _tiny_problem(seed=21, shared=True)
+    ref = O.moe_experts(x, logits, experts, top_k=2, shared=shared)
+    again = O.moe_experts(x, logits, experts, top_k=2, shared=shared, routed_h=(ref["hq"], ref["sh"]), shared_h=(ref["hsq"], ref["shs"]))
+    assert np.array_equal(again["out"], ref["out"]) and np.array_equal(again["y"], ref["y"])
+    other = ref["hq"].copy()
+    other[0, 0] ^= 0x08                                     # another exponent for one code
+    changed = O.moe_experts(x, logits, experts, top_k=2, shared=shared, routed_h=(other, ref["sh"]), shared_h=(ref["hsq"], ref["shs"]))
+    assert not np.array_equal(changed["y"][0], ref["y"][0]) and np.array_equal(changed["y"][1:], ref["y"][1:])
+    # the per-row form agrees with the whole-problem form and hands back what it computed
+    fetch = lambda e: {n: (q[e], s[e]) for n, (q, s) in experts.items()}
+    toks = [0, 3, x.shape[0] - 1]
+    rows = O.moe_experts_rows(x, toks, ref["indices"], ref["weights"], fetch, shared=shared, return_h=True)
+    assert np.array_equal(rows["out"], ref["out"][toks])
+    pos = ref["inv_perm"].reshape(-1, 2)[toks]
+    assert np.array_equal(rows["routed_h"][0], ref["hq"][pos]) and np.array_equal(rows["y"], ref["y"][pos])
+    assert np.array_equal(rows["ys"], ref["shared_out"][toks])
+    cont = O.moe_experts_rows(x, toks, ref["indices"], ref["weights"], fetch, shared=shared, routed_h=rows["routed_h"],
+                              shared_h=rows["shared_h"])
+    assert np.array_equal(cont, ref["out"][toks])
