@@ -139,6 +139,10 @@ MOE_API int moe_router_logits(const void* x_bf16, int M, int D, const void* w_ro
 MOE_API int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
                       uint8_t* xq, float* sx, moe_stream_t stream);
 
+/* moe.py:282 (`.astype(x.dtype)`) and the widening in front of the layer: elementwise f32 <-> bf16 conversion of n
+ * values (round-to-nearest-even towards bf16), so that a caller holding f32 activations needs no other library. */
+MOE_API int moe_convert(const void* src, int src_is_f32, void* dst, int dst_is_f32, long long n, moe_stream_t stream);
+
 /* The whole path (moe.py:97-114 + 225-232 + 281): router logits in, combined hidden
  * states out -- or, with w_router set, hidden states in (moe.py:235-282, moe_layer). */
 typedef struct MoeForwardArgs {

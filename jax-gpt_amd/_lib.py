@@ -60,6 +60,7 @@ SIGNATURES = {
     "moe_rmsnorm_quant": (_I, [_P, _P, _F, _I, _I, _P, _P, _P, _P]),
     "moe_router_workspace_bytes": (_Z, [_I, _I, _I]),
     "moe_router_logits": (_I, [_P, _I, _I, _P, _I, _P, _P, _P, _P, _Z, _P]),
+    "moe_convert": (_I, [_P, _I, _P, _I, C.c_longlong, _P]),
     "moe_forward_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I]),
     "moe_forward": (_I, [C.POINTER(MoeForwardArgs), _P, _Z, _P]),
 }

@@ -171,3 +171,25 @@ extern "C" int moe_quant_weight_block(const void* w, int src_is_f32, int E, int 
     hipLaunchKernelGGL(quant_weight_kernel<bf16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const bf16_t*)w, N, K, wq, sw);
   return moe_check_hip(hipGetLastError(), "quant_weight_block launch");
 }
+
+namespace {
+// f32 <-> bf16 conversion of a flat array (the layer computes from bf16 activations and returns its caller's
+// dtype, moe.py:282): round-to-nearest-even one way, exact the other
+__global__ __launch_bounds__(256) void convert_kernel(const void* __restrict__ src, int src_is_f32, void* __restrict__ dst,
+                                                     int dst_is_f32, long long n) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float v = src_is_f32 ? ((const float*)src)[i] : bf16_to_f32(((const bf16_t*)src)[i]);
+  if (dst_is_f32) ((float*)dst)[i] = v;
+  else ((bf16_t*)dst)[i] = f32_to_bf16(v);
+}
+}  // namespace
+
+extern "C" int moe_convert(const void* src, int src_is_f32, void* dst, int dst_is_f32, long long n, moe_stream_t stream) {
+  MOE_REQUIRE(n >= 0 && n < (1ll << 38), MOE_ERR_BAD_SHAPE, "convert: bad element count %lld", n);
+  MOE_REQUIRE(n == 0 || (src && dst), MOE_ERR_NULL, "convert: null pointer");
+  if (n == 0) return MOE_OK;
+  hipLaunchKernelGGL(convert_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, src, src_is_f32,
+                     dst, dst_is_f32, n);
+  return moe_check_hip(hipGetLastError(), "convert launch");
+}

@@ -13,6 +13,8 @@
 // (both may be empty), i.e. moe.py:235-282 with block.py:54-58 around it in one custom call.
 #include <cstdint>
 
+#include <hip/hip_runtime_api.h>   // hipStream_t (moe_hip.h itself is plain C and names no HIP type)
+
 #include "moe_hip.h"
 #include "xla/ffi/api/ffi.h"
 

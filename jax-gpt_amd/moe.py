@@ -11,7 +11,12 @@ Expert weights are block-scaled fp8 dicts ``{'w': (E, out, in) float8_e4m3fn,
 (quantize.py:31-42, model.py:89-97) with 128x128 scale blocks instead of
 per-row scales; real value = w * scale_inv (moe.py:29).  Plain (E, in, out)
 arrays, the reference's unquantised layout, are quantised on the GPU on first
-use.
+use.  The reference's own fp8 dicts (one scale per output row: experts
+``scale_inv (E, out, 1)``, dense layers ``(out, 1)``; quantize.py:18-42,
+model.py:79-114 with fp8=True) are accepted too: they are de-quantised once the way
+the reference's consumer of each does it (experts: w * scale_inv, moe.py:29; dense
+layers and the router: w / scale_inv, fp8.py:87-89) and re-quantised per 128x128
+block (a second rounding of the weights), cached for the life of the source tensor.
 """
 from __future__ import annotations
 
@@ -111,6 +116,18 @@ def permute(expert_indices, n_experts):
 # quantisers
 # ----------------------------------------------------------------------------
 
+def convert(t, dtype):
+    """f32 <-> bf16 conversion on the library's own kernel (round-to-nearest-even towards bf16)."""
+    if t.dtype == dtype:
+        return t
+    if {t.dtype, dtype} != {torch.float32, torch.bfloat16}:
+        raise TypeError(f"convert: f32 <-> bf16 only, got {t.dtype} -> {dtype}")
+    t = _dev(t, None, "t")
+    out = _empty(tuple(t.shape), dtype, t)
+    check(lib().moe_convert(_ptr(t), int(t.dtype == torch.float32), _ptr(out), int(dtype == torch.float32), t.numel(), _stream()))
+    return out
+
+
 def quant_act(x):
     """(R, K) bf16 -> (codes (R, K) float8_e4m3fn, scale_inv (R, K/128) f32)."""
     x = _dev(x, torch.bfloat16, "x")
@@ -156,50 +173,81 @@ def quantize_weight_block(w):
     return {"w": wq.view(torch.float8_e4m3fn), "scale_inv": sw}
 
 
-def block_fp8_from_per_row(d):
+def block_fp8_from_per_row(d, dense=False):
     """The reference's own fp8 dicts carry one scale per output row (`scale_inv` (E, out, 1) or (out, 1),
-    quantize.py:18-42).  This path computes with 128x128 blocks: de-quantise (w * scale_inv, moe.py:29) to f32
-    and quantise again per block.  A second rounding of the weights, so prefer quantising from bf16 where the
-    original weights exist."""
+    quantize.py:18-42).  This path computes with 128x128 blocks: de-quantise (experts: w * scale_inv, moe.py:29;
+    `dense` 2-D layers: w / scale_inv, fp8.py:87-89) to f32 and quantise again per block.  A second rounding of
+    the weights, so prefer quantising from bf16 where the original weights exist.  (The layer entry points do this
+    themselves, once per tensor, when handed such a dict.)"""
     q, s = d["w"], d["scale_inv"]
+    if not _per_row_scales(q, s):
+        raise ValueError(f"expected per-row scales {tuple(q.shape[:-1]) + (1,)}, got {tuple(s.shape)}")
+    wq, sw = _requantise_per_row(q, s, dense)
+    if q.dim() == 2:
+        wq, sw = wq[0], sw[0]
+    return {"w": wq.view(torch.float8_e4m3fn), "scale_inv": sw}
+
+
+_derived = {}
+
+
+def _cached(src, tag, build):
+    """Derived GPU copies (quantised weights, transposed router weights) are kept per source tensor and version,
+    and dropped when the source tensor is garbage-collected or has been modified in place."""
+    key = (tag, id(src))
+    hit = _derived.get(key)
+    if hit is not None and hit[0]() is src and hit[1] == src._version:
+        return hit[2]
+    val = build()
+    if hit is None or hit[0]() is not src:
+        weakref.finalize(src, _derived.pop, key, None)
+    _derived[key] = (weakref.ref(src), src._version, val)
+    return val
+
+
+def _per_row_scales(q, s):
+    """True for the reference's per-row layout: scale_inv (..., out, 1) next to w (..., out, in)."""
+    return s.dim() == q.dim() and s.shape[-1] == 1 and tuple(s.shape[:-1]) == tuple(q.shape[:-1])
+
+
+def _requantise_per_row(q, s, dense):
+    """De-quantise a per-row fp8 dict as its consumer in the reference does and quantise per 128x128 block."""
     if q.dtype != torch.float8_e4m3fn:
         q = _codes(q, "w").view(torch.float8_e4m3fn)
-    if s.shape[-1] != 1 or s.shape[:-1] != q.shape[:-1]:
-        raise ValueError(f"expected per-row scales {tuple(q.shape[:-1]) + (1,)}, got {tuple(s.shape)}")
-    w = _dev(q, None, "w").to(torch.float32) * _dev(s, None, "scale_inv").to(torch.float32)
-    return quantize_weight_block(w)
+    q = _dev(q, None, "w")
+    s = _dev(s, None, "scale_inv").to(torch.float32)
+    w = q.to(torch.float32) / s if dense else q.to(torch.float32) * s     # fp8.py:87-89 / moe.py:29
+    d = quantize_weight_block(w if w.dim() == 3 else w.unsqueeze(0))
+    return d["w"].view(torch.uint8), d["scale_inv"]
 
 
-_plain_cache = {}
-
-
-def _expert_weight(w, name):
-    """Accept a block-fp8 dict, or a plain (E, in, out) array as the reference stores
-    unquantised experts (model.py:98-101), which is transposed and quantised once."""
+def _expert_weight(w, name, dense=False):
+    """Accept a block-fp8 dict; a per-row fp8 dict of the reference (re-quantised per block once, cached); or a plain
+    (E, in, out) array as the reference stores unquantised experts (model.py:98-101), transposed and quantised
+    once.  `dense`: a 2-D layer of the shared expert, (in, out) plain or (out, in) fp8 (fp8.py:123-143).
+    Returns (codes (E, N, K) uint8, scale_inv (E, N/128, K/128) f32)."""
     if isinstance(w, dict) and "w" in w:
         q, s = w["w"], w["scale_inv"]
+        if _per_row_scales(q, s):
+            return _cached(q, ("per_row", dense, id(s), s._version), lambda: _requantise_per_row(q, s, dense))
         if q.dim() == 2:
             q, s = q.unsqueeze(0), s.unsqueeze(0)
         E, N, K = q.shape
         if tuple(s.shape) != (E, N // 128, K // 128):
             raise ValueError(
-                f"{name}: scale_inv has shape {tuple(s.shape)}; this path needs 128x128 block scales "
-                f"{(E, N // 128, K // 128)} (per-row scales of the reference's quantize.py must be re-quantised: "
-                "block_fp8_from_per_row(d), or quantize_weight_block on the bf16 weights)")
+                f"{name}: scale_inv has shape {tuple(s.shape)}; expected 128x128 block scales "
+                f"{(E, N // 128, K // 128)} or the reference's per-row scales {(E, N, 1)}")
         return _codes(q, name + "['w']"), _dev(s, torch.float32, name + "['scale_inv']")
     if not isinstance(w, torch.Tensor):
         raise TypeError(f"{name}: expected a tensor or an fp8 dict")
-    key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
-    hit = _plain_cache.get(key)
-    if hit is not None and hit[0]() is w:
-        return hit[1], hit[2]
-    w3 = w.unsqueeze(0) if w.dim() == 2 else w
-    if w3.dtype not in (torch.bfloat16, torch.float32):
-        w3 = w3.to(torch.float32)
-    d = quantize_weight_block(w3.transpose(-1, -2).contiguous())      # (E, in, out) -> (E, out, in)
-    q, s = d["w"].view(torch.uint8), d["scale_inv"]
-    _plain_cache[key] = (weakref.ref(w), q, s)
-    return q, s
+
+    def build():
+        w3 = w.unsqueeze(0) if w.dim() == 2 else w
+        if w3.dtype not in (torch.bfloat16, torch.float32):
+            w3 = w3.to(torch.float32)
+        d = quantize_weight_block(w3.transpose(-1, -2).contiguous())      # (E, in, out) -> (E, out, in)
+        return d["w"].view(torch.uint8), d["scale_inv"]
+    return _cached(w, "plain", build)
 
 
 # ----------------------------------------------------------------------------
@@ -297,27 +345,28 @@ def shared_expert_forward(x, gate_proj, up_proj, down_proj):
     return gemm_down(hq, sh, down_proj, off)
 
 
-_router_cache = {}
-
-
 def _router_weight(w, name):
     """The reference keeps router weights input-major, (D, E) / (D, 1) (model.py:83-85, used as x @ w at
-    moe.py:50 and :278); the kernel wants them K-contiguous, (E, D) bf16: transposed once and cached."""
-    if isinstance(w, dict):
-        raise TypeError(f"{name}: an fp8 router weight is not supported; pass the bf16/f32 (D, E) array")
+    moe.py:50 and :278); the kernel wants them K-contiguous, (E, D) bf16: transposed once and cached.  The fp8 form
+    of the reference ({'w': (E, D) e4m3, 'scale_inv': (E, 1)}, model.py:107 with fp8=True) is de-quantised once to
+    bf16 as fp8.py:87-89 does (w / scale_inv); the matmul then runs in bf16 on f32 accumulators, where the reference
+    also quantises the activations per row (fp8.py:30-45)."""
+    if isinstance(w, dict) and "w" in w:
+        q, sc = w["w"], w["scale_inv"]
+        if q.dim() != 2 or not _per_row_scales(q, sc):
+            raise ValueError(f"{name}: expected {{'w': (out, in) e4m3, 'scale_inv': (out, 1)}}, got {tuple(q.shape)} / {tuple(sc.shape)}")
+
+        def deq():
+            qq = q if q.dtype == torch.float8_e4m3fn else _codes(q, name).view(torch.float8_e4m3fn)
+            return (_dev(qq, None, name).to(torch.float32) / _dev(sc, None, name).to(torch.float32)).to(torch.bfloat16).contiguous()
+        return _cached(q, ("router_fp8", id(sc), sc._version), deq)
     if not isinstance(w, torch.Tensor):
-        raise TypeError(f"{name}: expected a tensor")
+        raise TypeError(f"{name}: expected a tensor or an fp8 dict")
     if not w.is_cuda:
         raise RuntimeError(f"{name}: must live on the GPU (this path has no CPU fallback)")
     if w.dim() != 2 or w.dtype not in (torch.bfloat16, torch.float32):
         raise TypeError(f"{name}: expected a 2-D bf16/f32 array (D, E), got {tuple(w.shape)} {w.dtype}")
-    key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
-    hit = _router_cache.get(key)
-    if hit is not None and hit[0]() is w:
-        return hit[1]
-    wt = w.t().to(torch.bfloat16).contiguous()
-    _router_cache[key] = (weakref.ref(w), wt)
-    return wt
+    return _cached(w, "router", lambda: w.t().to(torch.bfloat16).contiguous())
 
 
 def router_logits(x, gate_weight, shared_expert_gate_weight=None):
@@ -328,12 +377,12 @@ def router_logits(x, gate_weight, shared_expert_gate_weight=None):
     E, D = wr.shape
     M = x.shape[0]
     if x.shape[1] != D:
-        raise ValueError(f"gate_weight: expected ({x.shape[1]}, E), got {tuple(gate_weight.shape)}")
+        raise ValueError(f"gate_weight: expected ({x.shape[1]}, E), got a weight for hidden size {D}")
     wsg = None
     if shared_expert_gate_weight is not None:
         wsg = _router_weight(shared_expert_gate_weight, "shared_expert_gate_weight")
         if tuple(wsg.shape) != (1, D):
-            raise ValueError(f"shared_expert_gate_weight: expected ({D}, 1), got {tuple(shared_expert_gate_weight.shape)}")
+            raise ValueError(f"shared_expert_gate_weight: expected ({D}, 1), got a weight for {tuple(wsg.shape)[::-1]}")
     logits = _empty((M, E), torch.float32, x)
     gate = _empty((M,), torch.float32, x) if wsg is not None else None
     nbytes = lib().moe_router_workspace_bytes(M, D, E)
@@ -385,9 +434,9 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     if logits is not None and tuple(logits.shape) != (M, E):
         raise ValueError(f"router_logits: expected {(M, E)}, got {tuple(logits.shape)}")
     if wr is not None and tuple(wr.shape) != (E, D):
-        raise ValueError(f"gate_weight: expected {(D, E)}, got {tuple(gate_weight.shape)}")
+        raise ValueError(f"gate_weight: expected {(D, E)} (or its fp8 form ({E}, {D})), got a weight for {tuple(wr.shape)[::-1]}")
     if wsg is not None and tuple(wsg.shape) != (1, D):
-        raise ValueError(f"shared_expert_gate_weight: expected {(D, 1)}, got {tuple(shared_expert_gate_weight.shape)}")
+        raise ValueError(f"shared_expert_gate_weight: expected {(D, 1)}, got a weight for {tuple(wsg.shape)[::-1]}")
     if wsg is not None and shared is None:
         raise ValueError("shared_expert_gate_weight needs a shared expert")
     if wg.shape != (E, I, D) or wu.shape != (E, I, D) or wd.shape != (E, D, I):
@@ -418,9 +467,9 @@ def moe_experts(x, router_logits, *, top_k, experts, routing="softmax", bias=Non
     a.sw_gate, a.sw_up, a.sw_down = sg.data_ptr(), su.data_ptr(), sd.data_ptr()
     SI = 0
     if shared is not None:
-        swg, ssg = _expert_weight(shared["gate_proj"], "shared gate_proj")
-        swu, ssu = _expert_weight(shared["up_proj"], "shared up_proj")
-        swd, ssd = _expert_weight(shared["down_proj"], "shared down_proj")
+        swg, ssg = _expert_weight(shared["gate_proj"], "shared gate_proj", dense=True)
+        swu, ssu = _expert_weight(shared["up_proj"], "shared up_proj", dense=True)
+        swd, ssd = _expert_weight(shared["down_proj"], "shared down_proj", dense=True)
         SI = swg.shape[1]
         if swg.shape != (1, SI, D) or swu.shape != (1, SI, D) or swd.shape != (1, D, SI):
             raise ValueError("shared expert weight shapes do not fit")
@@ -482,8 +531,10 @@ def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=
         raise ValueError(f"x: expected (B, T, D), got {tuple(x.shape)}")
     B, T, D = x.shape
     x_flat = x.reshape(B * T, D)
-    if x_flat.dtype != torch.bfloat16:
-        x_flat = x_flat.to(torch.bfloat16)          # the path computes from bf16 activations
+    if x_flat.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"x: expected bf16 or f32 activations, got {x.dtype}")
+    if x_flat.dtype == torch.float32:               # the path computes from bf16 activations
+        x_flat = convert(_dev(x_flat, torch.float32, "x"), torch.bfloat16)
     shared = None
     if params.get("shared_gate_proj") is not None:
         shared = dict(gate_proj=params["shared_gate_proj"], up_proj=params["shared_up_proj"],
@@ -494,4 +545,6 @@ def moe_layer(x, params, n_experts_per_token, n_devices=1, axis_name="tp", mesh=
                       routing="softmax", shared=shared, gate_weight=params["gate_weight"],
                       shared_expert_gate_weight=params.get("shared_expert_gate_weight") if shared is not None else None,
                       norm_weight=_norm_weight, norm_eps=_norm_eps, add_residual=_add_residual)
-    return out.reshape(B, T, D).to(x.dtype)
+    if x.dtype == torch.float32:                    # moe.py:282: back to the caller's dtype
+        out = convert(out, torch.float32)
+    return out.reshape(B, T, D)

@@ -552,9 +552,9 @@ def test_empty_batch_and_limits(jg):
         jg.route_softmax_topk(H.to_cuda(rng.standard_normal((2, 1025), dtype=np.float32)), 2)
 
 
-def test_per_row_fp8_dicts_are_converted_on_request(jg):
-    """The reference's fp8 format (one scale per output row, quantize.py:18-42) is refused by the GEMMs with a
-    message and converted by block_fp8_from_per_row: de-quantise as moe.py:29 does, quantise per 128 x 128 block."""
+def test_per_row_fp8_dicts_are_converted(jg):
+    """The reference's fp8 format (one scale per output row, quantize.py:18-42) is converted once, by the entry
+    points themselves or by block_fp8_from_per_row: de-quantise as moe.py:29 does, quantise per 128 x 128 block."""
     import torch
     _say("per-row fp8 dicts")
     E, N, K = 2, 128, 256
@@ -566,8 +566,8 @@ def test_per_row_fp8_dicts_are_converted_on_request(jg):
     d = {"w": q, "scale_inv": scale_inv}
     off = torch.tensor([0, 8, 16], dtype=torch.int32, device="cuda")
     xq, sx = jg.quant_act(torch.randn(16, K, device="cuda", generator=g).to(torch.bfloat16))
-    with pytest.raises(ValueError, match="block_fp8_from_per_row"):
-        jg.gemm_gateup_swiglu(xq, sx, d, d, off)
+    with pytest.raises(ValueError, match="block scales"):
+        jg.gemm_gateup_swiglu(xq, sx, {"w": q, "scale_inv": scale_inv[:, :, 0]}, d, off)
     b = jg.block_fp8_from_per_row(d)
     assert b["w"].shape == (E, N, K) and b["scale_inv"].shape == (E, 1, 2)
     deq_row = q.float() * scale_inv
@@ -575,6 +575,8 @@ def test_per_row_fp8_dicts_are_converted_on_request(jg):
     assert (deq_blk - deq_row).abs().max() <= 0.07 * deq_row.abs().max()    # one more e4m3 rounding
     hq, sh = jg.gemm_gateup_swiglu(xq, sx, b, b, off)
     assert hq.shape == (16, N) and torch.isfinite(sh).all()
+    hq2, sh2 = jg.gemm_gateup_swiglu(xq, sx, d, d, off)                     # the per-row dict itself, converted on the way in
+    assert torch.equal(hq.view(torch.uint8), hq2.view(torch.uint8)) and torch.equal(sh, sh2)
 
 
 @pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
