@@ -25,9 +25,23 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP8_TFLOPS = 5000.0     # MI355X dense fp8 MFMA (published)
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E (published)
-# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# file (counter x calibration factor; the summary and the commands are in profiles/).  None = not measured.
-MEASURED_TRAFFIC = {"deepseek_v3_prefill": 8757e6 + 146e6}
+
+
+def measured_traffic(workload):
+    """HBM-side bytes per launch of the workload's dominant kernel (the routed gate/up grouped GEMM), as measured
+    with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: read at run time from the committed summary under profiles/,
+    which carries the commands and the calibration next to a line
+        traffic: workload=<name> kernel=gateup_routed fetch_bytes=<n> write_bytes=<n>
+    Returns (bytes or None, the file it came from or None)."""
+    import glob
+    import re
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic*.txt"))):
+        for ln in open(path):
+            m = re.match(r"\s*traffic:\s+workload=(\S+)\s+kernel=gateup_routed\s+fetch_bytes=(\d+)\s+write_bytes=(\d+)", ln)
+            if m and m.group(1) == workload:
+                return float(m.group(2)) + float(m.group(3)), os.path.relpath(path, ROOT)
+    return None, None
+
 
 WORKLOADS = {
     # benchmark configs 3 and 4 (BASELINE.json): DeepSeek-V3-style layer
@@ -163,6 +177,53 @@ def run_workload(jg, torch, name, cfg, layer, steps, warmup):
     return res
 
 
+def run_ep_shard(jg, torch, steps, warmup, seed=5):
+    """Benchmark config 5: one GPU's expert-parallel shard.  32 local experts of the DeepSeek-V3 shape receive
+    16384 pre-dispatched rows (already in expert order: row_ids = NULL), group sizes from Zipf(1.2) with empty
+    experts, combine with top-8 weights from Dirichlet(1) into 2048 tokens.  A step = gate/up GEMM, down GEMM,
+    combine."""
+    import numpy as np
+    E, D, I, k, M = 32, 7168, 2048, 8, 2048
+    R = M * k
+    rng = np.random.Generator(np.random.Philox(seed))
+    p = 1.0 / np.arange(1, E + 1) ** 1.2
+    p[[5, 17, 30]] = 0.0                                       # forced empty experts
+    p /= p.sum()
+    group_sizes = np.bincount(rng.choice(E, size=R, p=p), minlength=E).astype(np.int32)
+    off = torch.from_numpy(np.concatenate([[0], np.cumsum(group_sizes)]).astype(np.int32)).cuda()
+    weights = torch.from_numpy(rng.dirichlet(np.ones(k), size=M).astype(np.float32)).cuda()
+    inv_perm = torch.from_numpy(rng.permutation(R).astype(np.int32)).cuda()
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    experts = dict(gate_proj=make_weights(jg, torch, E, I, D, gen), up_proj=make_weights(jg, torch, E, I, D, gen),
+                   down_proj=make_weights(jg, torch, E, D, I, gen))
+    xq, sx = jg.quant_act(torch.randn((R, D), dtype=torch.float32, device="cuda", generator=gen).to(torch.bfloat16))
+    log(f"ep_shard_skewed: rows per expert, ascending: {sorted(int(v) for v in group_sizes)}")
+
+    def step():
+        hq, sh = jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], off)
+        y = jg.gemm_down(hq, sh, experts["down_proj"], off)
+        return jg.combine(y, weights, inv_perm)
+
+    out = step()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all(), "non-finite output"
+    ms, _ = timed(torch, step, steps, warmup)
+    k_ms, _ = timed(torch, lambda: jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], off), steps,
+                    max(2, warmup // 2))
+    flops = 6.0 * R * D * I
+    k_flops = 4.0 * R * D * I
+    touched = int((group_sizes > 0).sum())
+    return {"metric": "expert-parallel shard fp8 TFLOP/s (pre-dispatched rows, gate/up + down + combine)",
+            "value": flops / ms / 1e9, "unit": "TFLOP/s", "ms_per_step": ms, "frac_of_peak": flops / ms / 1e9 / PEAK_FP8_TFLOPS,
+            "config": {"workload": "ep_shard_skewed", "local_experts": E, "rows": R, "D": D, "I": I, "k": k, "tokens": M,
+                       "touched_experts": touched, "largest_group": int(group_sizes.max()), "group_sizes": "Zipf(1.2)"},
+            "roofline": {"bound": "mfma", "achieved": k_flops / k_ms / 1e9, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                         "frac": k_flops / k_ms / 1e9 / PEAK_FP8_TFLOPS, "traffic": None,
+                         "kernel": "grouped_gemm_classes_kernel<0> (gate/up + SwiGLU + h quantisation), rows in expert order",
+                         "avg_launch_ms": k_ms, "flops_per_launch": k_flops}}
+
+
 def cpu_baseline(cfg, seconds_budget=25.0):
     """The reference's dataflow (oracle/reference_dataflow.py, a port) on the host cores, on a bounded
     sample of the prefill workload: a few experts at their mean row count."""
@@ -187,6 +248,7 @@ def main():
     ap.add_argument("--workload", default="deepseek_v3_prefill", choices=sorted(WORKLOADS))
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-extra", action="store_true", help="skip the Qwen3-MoE prefill and the expert-parallel shard parts")
     ap.add_argument("--bias-std", type=float, default=0.1,
                     help="standard deviation of the selection bias of sigmoid_grouped routing (0.1 = the workload as "
                          "specified: the same 7 of 8 groups win almost every token; 0 = balanced routing)")
@@ -220,6 +282,16 @@ def main():
         dcfg = WORKLOADS["deepseek_v3_decode"]
         decode = run_workload(jg, torch, "deepseek_v3_decode", dcfg, layer, max(args.steps, 20), args.warmup)
         log(json.dumps(decode))
+    # the other two MFMA-bound configurations of the benchmark, measured in the same run (the default run only)
+    qwen3 = ep_shard = None
+    if args.workload == "deepseek_v3_prefill" and not args.no_extra:
+        del layer
+        torch.cuda.empty_cache()
+        qcfg = WORKLOADS["qwen3_moe_prefill"]
+        qwen3 = run_workload(jg, torch, "qwen3_moe_prefill", qcfg, make_layer(jg, torch, qcfg, seed=2), max(args.steps, 20), args.warmup)
+        log(json.dumps(qwen3))
+        ep_shard = run_ep_shard(jg, torch, max(args.steps, 20), args.warmup)
+        log(json.dumps(ep_shard))
 
     gk = main_res["gateup_kernel"]
     if is_decode:
@@ -229,9 +301,10 @@ def main():
                 "avg_launch_ms": gk["avg_launch_ms"]}
     else:
         metric, value, unit = "MoE layer fp8 TFLOP/s (prefill)", main_res["tflops"], "TFLOP/s"
+        traffic, traffic_src = measured_traffic(args.workload) if args.bias_std == 0.1 else (None, None)
         roof = {"bound": "mfma", "achieved": gk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": MEASURED_TRAFFIC.get(args.workload) if args.bias_std == 0.1 else None,
-                "kernel": "grouped_gemm_kernel<0, 2>, routed launch (gate/up + SwiGLU + h quantisation)",
+                "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
+                "kernel": "grouped_gemm_classes_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
                 "algorithmic_bytes_per_launch": gk["bytes_per_launch"],
                 "avg_launch_ms": gk["avg_launch_ms"], "flops_per_launch": gk["flops_per_launch"]}
     line = {
@@ -251,8 +324,24 @@ def main():
                           "graph_replay_value": decode.get("graph_gbs"), "touched_experts": decode["touched_experts"],
                           "weight_bytes": decode["weight_bytes"], "frac_of_peak": decode["gbs"] / PEAK_HBM_GBS,
                           "roofline": {"bound": "hbm", "achieved": dk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": dk["gbs"] / PEAK_HBM_GBS, "traffic": None,
+                                       "frac": dk["gbs"] / PEAK_HBM_GBS,
+                                       "traffic": measured_traffic("deepseek_v3_decode")[0],
+                                       "traffic_source": measured_traffic("deepseek_v3_decode")[1],
+                                       "algorithmic_bytes_per_launch": dk["bytes_per_launch"],
+                                       "kernel": "grouped_gemm_kernel<0, 0>, routed launch (gate/up + SwiGLU + h quantisation)",
                                        "avg_launch_ms": dk["avg_launch_ms"]}}
+    if qwen3:
+        qk = qwen3["gateup_kernel"]
+        line["qwen3_moe_prefill"] = {"metric": "MoE layer fp8 TFLOP/s (prefill)", "value": qwen3["tflops"], "unit": "TFLOP/s",
+                                     "ms_per_step": qwen3["ms_per_step"], "frac_of_peak": qwen3["tflops"] / PEAK_FP8_TFLOPS,
+                                     "config": {"workload": "qwen3_moe_prefill", **{k: WORKLOADS["qwen3_moe_prefill"][k] for k in ("M", "D", "E", "k", "I", "SI", "routing")},
+                                                "touched_experts": qwen3["touched_experts"]},
+                                     "roofline": {"bound": "mfma", "achieved": qk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                                                  "frac": qk["tflops"] / PEAK_FP8_TFLOPS, "traffic": None,
+                                                  "kernel": "grouped_gemm_classes_kernel<0>, routed launch", "avg_launch_ms": qk["avg_launch_ms"],
+                                                  "flops_per_launch": qk["flops_per_launch"]}}
+    if ep_shard:
+        line["ep_shard_skewed"] = ep_shard
     if not args.no_cpu:
         pcfg = cfg if not is_decode else WORKLOADS["deepseek_v3_prefill"]
         line["cpu_baseline"] = cpu_baseline(pcfg)
