@@ -248,10 +248,9 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   if (rc) return join(rc);
   // the permutation kernels also list the routed GEMMs' row tiles (they hold every expert's row range anyway)
   TileList tiles;
-  int bm = 0;
-  if ((rc = moe_gemm_tile_list(R, a->E, b.gemm_ws, b.gemm_ws_bytes, &tiles, &bm))) return join(rc);
+  if ((rc = moe_gemm_tile_list(R, a->E, b.gemm_ws, b.gemm_ws_bytes, &tiles))) return join(rc);
   if ((rc = moe_permute_impl(idx, a->M, a->k, a->E, gsz, b.group_offsets, stid, nullptr, inv, b.permute_ws,
-                             b.permute_ws_bytes, tiles, bm, stream)))
+                             b.permute_ws_bytes, tiles, stream)))
     return join(rc);
   if (!quant_joined) {
     if (rc_shared) return join(rc_shared);

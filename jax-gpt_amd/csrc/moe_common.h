@@ -50,28 +50,61 @@ struct TileList {
   TileHeader* hdr;
   TileEntry* tiles;
 };
-// An expert with `rows` rows gets ceil(rows / bm) row tiles (bm = 32 or 256) whose heights, counted in units of 32
-// rows (16 for bm = 32), differ by at most one: no tile computes more than one unit of padding, and tiles that
-// share a weight slab take about the same time per K step and walk it together, so the later reader finds it in L2.
-__host__ __device__ inline int moe_tile_count(int rows, int bm) {
-  if (rows <= 0) return 0;
-  return bm == 256 ? (rows + 255) >> 8 : (rows + 31) >> 5;
-}
+// An expert with `rows` rows gets ceil(rows / 256) row tiles whose heights, counted in units of 32 rows, differ by
+// at most one: no tile computes more than 31 rows of padding, and tiles that share a weight slab take about the same
+// time per K step and walk it together, so the later reader finds it in L2.
+__host__ __device__ inline int moe_tile_count(int rows) { return rows <= 0 ? 0 : (rows + 255) >> 8; }
 // first row (relative to the expert's first) and row count of tile t of nt
-__host__ __device__ inline void moe_tile_span(int rows, int bm, int nt, int t, int& start, int& count) {
+__host__ __device__ inline void moe_tile_span(int rows, int nt, int t, int& start, int& count) {
   if (nt == 1) {   // (integer division costs some forty instructions on this hardware: the one-tile case takes none)
     start = 0;
     count = rows;
     return;
   }
-  const int ushift = bm == 256 ? 5 : 4;
-  const int units = (rows + (1 << ushift) - 1) >> ushift;
+  const int units = (rows + 31) >> 5;
   const int base = units / nt, extra = units - base * nt;
-  const int u0 = t * base + (t < extra ? t : extra);
-  start = u0 << ushift;
-  const int full = (base + (t < extra ? 1 : 0)) << ushift;
+  start = (t * base + (t < extra ? t : extra)) << 5;
+  const int full = (base + (t < extra ? 1 : 0)) << 5;
   count = full < rows - start ? full : rows - start;
 }
+#ifdef __HIPCC__
+// Where an expert's tiles go in the work list.  The grouped GEMM deals contiguous eighths of the list to the 8 XCDs
+// (tiles that share a weight slab then share an L2), so the eighths should cost about the same: with group sizes
+// as skewed as a biased router makes them, natural expert order leaves one XCD with up to a tenth more work than the
+// average, and the launch ends with its slowest XCD.  The experts are therefore ranked by size (ties: lower index
+// first) and dealt to eight bins in snake order (0..7, 7..0, ...); the list holds bin after bin, each bin's
+// experts largest first.
+// Called by every thread of a workgroup with at least E threads; thread e owns expert e (rows = 0 for e >= E);
+// lds_rows and lds_key are int[blockDim.x] arrays in LDS.  Returns the index of expert e's first tile and, in
+// *total_tiles, the length of the list.
+__device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int* lds_key, int* total_tiles) {
+  lds_rows[e] = e < E ? rows : 0;
+  __syncthreads();
+  int key = e;
+  if (e < E) {
+    int rank = 0;
+#pragma unroll 8
+    for (int o = 0; o < E; ++o) {
+      const int r = lds_rows[o];
+      rank += (r > rows || (r == rows && o < e)) ? 1 : 0;
+    }
+    const int round = rank >> 3, posn = rank & 7;
+    key = ((round & 1) ? 7 - posn : posn) * 128 + round;   // E <= 1024: at most 128 rounds
+  }
+  lds_key[e] = key;
+  __syncthreads();
+  int first = 0, total = 0;
+#pragma unroll 8
+  for (int o = 0; o < E; ++o) {
+    const int t = moe_tile_count(lds_rows[o]);
+    total += t;
+    first += lds_key[o] < key ? t : 0;
+  }
+  *total_tiles = total;
+  return first;
+}
+#endif
+
 // Where the routing kernels take a token's logits from: an (M, E) array, or the router matmul's split-K partial
 // sums [splits][M][N] (N = E, + 1 when the shared expert's gate is the last column), which they add in slice order
 // and round to bf16 themselves -- the logits then never travel through memory unless out_logits asks for them.
@@ -93,10 +126,10 @@ int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, in
 // grouped GEMMs with an optional pre-built tile list in ws (moe_gemm.hip); the extern "C" entry points build their
 // own.  moe_gemm_tile_list describes the list the GEMMs of (R rows, E experts) expect in ws, so that the permutation
 // kernels, which hold every expert's row range anyway, can write it (moe_permute_impl) and no launch is spent on it.
-int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list, int* bm);
+int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list);
 int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_sizes, int32_t* group_offsets,
                      int32_t* sorted_token_ids, int32_t* sort_order, int32_t* inv_perm, void* ws, size_t ws_bytes,
-                     TileList tiles, int bm, moe_stream_t stream);
+                     TileList tiles, moe_stream_t stream);
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
                          const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
                          int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,

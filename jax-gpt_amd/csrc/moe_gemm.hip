@@ -15,38 +15,39 @@
 // activation fragment its column operand, so a lane holds four weight rows of
 // ONE activation row: one activation scale per lane per fragment, not four.
 //
-// Data movement.  A workgroup (8 waves, two per SIMD) owns a work item =
-// (expert, <= BM activation rows, 256 weight rows) and walks K in steps of 128
-// through a ring of LDS stages.  Tiles are copied global -> LDS by
+// Data movement.  A workgroup (8 waves, two per SIMD, one workgroup per CU) owns a
+// work item = (expert, <= 256 activation rows, 256 weight rows) and walks K in
+// steps of 128 through a ring of LDS stages.  Tiles are copied global -> LDS by
 // global_load_lds (no registers in between) ahead of their use.  In
 // MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of the
 // same output columns, so silu(g)*u is lane-local and the 1x128 amax stays
 // inside the workgroup.  Waves form a 4 x 2 grid: wave (wi, xj) owns weight rows
 // {32wi..32wi+31} of each half (GATEUP) or {64wi..64wi+63} (DOWN) against the
 // 16-row activation fragments 2j + xj (alternating between the two wave sets, so
-// a short tile still splits evenly).  Three tile heights are built:
-//   BM = 32:  wave tile 64 x 16, two stages of 36 KB, TWO workgroups per CU: for batches of a few rows per
-//             expert the kernel only streams weights, and a second workgroup keeps the stream going while
-//             the first starts or finishes a work item;
-//   BM = 128: wave tile 64 x 64, three stages of 48.5 KB (copies two steps ahead);
-//   BM = 256: wave tile 64 x 128, two stages of 65 KB (copies one, twice as long,
-//             step ahead); half the weight traffic, LDS reads and barriers per MFMA.
+// a short tile still splits evenly).
 //
-// The copies of a step are issued a few at a time between MFMA groups, not in
-// one burst, and the two waves of each SIMD run out of phase (see the K loop).
+// What bounds a work item.  One CU draws at most about 22 GB/s from HBM and about
+// 85 GB/s from its XCD's L2 through its vector L1, however many copies it keeps in
+// flight (measured with a streaming workgroup of this kernel's copy pattern; all
+// 256 CUs together reach the HBM rate).  A K step of a full tile moves 64 KB into
+// LDS and holds 2048 matrix-core cycles per SIMD: the activation tile is shared by
+// the item's 16 column blocks and comes from L2, the weight tile comes from L2 when
+// a neighbouring row tile of the same expert has just fetched it and from HBM
+// otherwise (always, for an expert of one row tile).  An expert of few rows is
+// therefore a weight stream at the per-CU HBM rate whatever the kernel does with
+// its rows; the kernel's part is to keep that stream and the large experts'
+// matrix work going side by side on different CUs, and to waste neither.
 //
-// Row tiles are listed on the device by build_tiles_kernel (no host read-back
-// of group sizes); a workgroup's work item is a (row tile, column block) pair
-// derived from its index, in [expert][column block][row tile] order, and the
-// items are dealt to the 8 XCDs in contiguous ranges, so the row tiles and
-// column blocks that share a weight slab or an activation tile run together
-// under one L2.  An expert's rows are cut into tiles of equal height, so that
-// the tiles sharing a weight slab advance at the same pace.
+// Row tiles are listed on the device (build_tiles_kernel here, or the permutation
+// kernels inside moe_forward: no host read-back of group sizes); a workgroup's
+// work item is a (row tile, column block) pair derived from its index, in
+// [expert][column block][row tile] order, and the items are dealt to the 8 XCDs in
+// contiguous ranges, so the row tiles and column blocks that share a weight slab
+// or an activation tile run together under one L2.
 #include <stdlib.h>
 
-#include <type_traits>
-
 #include <mutex>
+#include <type_traits>
 
 #include "moe_common.h"
 
@@ -62,43 +63,35 @@ constexpr int NWAVES = 8;
 constexpr int NT = 64 * NWAVES;
 constexpr int MODE_GATEUP = 0;
 constexpr int MODE_DOWN = 1;
+constexpr int MAX_KB = 256;   // K <= 32768
+constexpr int W_TILE_BYTES = BW * BK;   // 32 KB
+constexpr int ROTC = 2;       // MFMA groups by which wave set 1 trails wave set 0 (measured: 1 to 3 within 2 %)
 
 // ---- work list -----------------------------------------------------------
 
-// One workgroup lists the row tiles of every expert, [expert][tile]; thread e owns expert e.
-__global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __restrict__ group_offsets, int E, int bm,
+// One workgroup lists the row tiles of every expert (an expert's tiles side by side; which expert where: see
+// moe_tile_first); thread e owns expert e.
+__global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __restrict__ group_offsets, int E,
                                                           TileList l) {
-  __shared__ int wave_tot[16];
+  __shared__ int s_rows[1024];
+  __shared__ int s_key[1024];
   const int e = threadIdx.x;
-  const int lane = e & 63, wv = e >> 6;
   int start = 0, rows = 0;
   if (e < E) {
     start = group_offsets[e];
     rows = group_offsets[e + 1] - start;
   }
-  const int tiles = moe_tile_count(rows, bm);
-  int incl = tiles;
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    int o = __shfl_up(incl, off, MOE_WAVE);
-    if (lane >= off) incl += o;
-  }
-  if (lane == 63) wave_tot[wv] = incl;
-  __syncthreads();
-  int wbase = 0, total = 0;
-  for (int i = 0; i < 16; ++i) {
-    if (i < wv) wbase += wave_tot[i];
-    total += wave_tot[i];
-  }
-  const int first = wbase + incl - tiles;
+  const int tiles = moe_tile_count(rows);
+  int total = 0;
+  const int first = moe_tile_first(e, E, rows, s_rows, s_key, &total);
   for (int t = 0; t < tiles; ++t)
     if (first + t < l.max_tiles) l.tiles[first + t] = TileEntry{e, start, rows, first};   // (cannot overflow for consistent offsets)
   if (e == 0) l.hdr->n_tiles = total < l.max_tiles ? total : l.max_tiles;
 }
 
-// ---- main kernel ---------------------------------------------------------
+// ---- the kernel ------------------------------------------------------------------------------------------------
 //
-// LDS stage = [weight tile 256 x 128 B][activation tile BM x 128 B][BM activation scales].
+// LDS stage = [weight tile 256 x 128 B][activation tile 32 XF x 128 B][32 XF activation scales].
 // Tiles are row-major with 128-byte rows; the 16-byte chunk c of row r sits at chunk position
 // c ^ ((r >> 1) & 7).  A fragment lane (row fr = lane % 16, quarter fq = lane / 16) feeds the
 // MFMA with K bytes [16 fq, +16) and [64 + 16 fq, +16) of its row -- the same choice for both
@@ -108,409 +101,10 @@ __global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __rest
 // consecutive tile rows; the swizzle is applied by choosing which 16-byte piece of the row
 // each lane fetches.  No asynchronous load ever targets a register.
 
-constexpr int MAX_KB = 256;   // K <= 32768
-constexpr int W_TILE_BYTES = BW * BK;   // 32 KB
-
-template <int XW>   // XW = 0: BM = 32 (two workgroups per CU), XW = 1: BM = 128, XW = 2: BM = 256
-struct Cfg {
-  static constexpr int BM = XW == 0 ? 32 : 128 * XW;
-  static constexpr int XF = BM / 32;                           // activation fragments per wave
-  static constexpr int WG_PER_CU = XW == 0 ? 2 : 1;
-  static constexpr int NSTAGE = XW == 1 ? 3 : 2;
-  static constexpr int PRE = NSTAGE - 1;                       // copies run PRE steps ahead
-  static constexpr int X_TILE_BYTES = BM * BK;
-  static constexpr int STAGE_X_OFF = W_TILE_BYTES;
-  static constexpr int STAGE_S_OFF = W_TILE_BYTES + X_TILE_BYTES;
-  static constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4;
-  static constexpr int WSCALE_OFF = NSTAGE * STAGE_BYTES;      // [2][MAX_KB] weight block scales of the work item
-  static constexpr int RING_BYTES = WSCALE_OFF + 2 * MAX_KB * 4;
-  static constexpr int EPI_BYTES = BM * 512;                   // bf16 staging of MODE_DOWN (<= RING_BYTES)
-  static constexpr int LDS_BYTES = RING_BYTES > EPI_BYTES ? RING_BYTES : EPI_BYTES;   // 76032 / 151040 / 133120
-  static constexpr int X_DMA = XW == 0 ? 1 : 2 * XW;           // 1 KB activation row groups per wave per step
-                                                               // (at BM = 32 only waves 0-3 have one: see XSKIP)
-  static constexpr int VM_PER_STEP = 4 + X_DMA + 1;            // + 4 weight row groups + 1 scale copy
-  // skip the copies of activation rows past the end of a short tile; only where every step waits for all of its
-  // copies anyway (PRE == 1), so that no wait has to count a varying number of them
-  static constexpr bool XSKIP = PRE == 1;
-  // MFMA groups by which wave set 1 trails wave set 0 (build-time tuning knobs; measured best: half a step at
-  // BM = 128, two of the eight groups at BM = 256, where registers allow no more)
-#ifndef MOE_ROT1
-#define MOE_ROT1 2
-#endif
-#ifndef MOE_ROT2
-#define MOE_ROT2 2
-#endif
-  static constexpr int ROT = XW == 0 ? 0 : XW == 1 ? MOE_ROT1 : MOE_ROT2;
-};
-
-// Sched<XW>::first(j) = index of the first copy operation issued after MFMA group j (first(XF) = VM_PER_STEP).
-// The copies of a step are spread over its first XF * NUM / 4 groups (build-time tuning knobs MOE_SCHED1 /
-// MOE_SCHED2 = NUM for BM = 128 / 256; 0 = all copies at the start of the step, 4 = spread over the whole step).
-// Measured best: three quarters of the step at BM = 128 (copies run two steps ahead there), the first half at
-// BM = 256 (one step ahead: the later a copy is issued, the less time it has to land).
-#ifndef MOE_SCHED1
-#define MOE_SCHED1 3
-#endif
-#ifndef MOE_SCHED2
-#define MOE_SCHED2 2
-#endif
-#ifndef MOE_FENCE
-#define MOE_FENCE 1
-#endif
-#ifndef MOE_ROTC
-#define MOE_ROTC 2   // MFMA groups by which wave set 1 trails wave set 0 in the tile-class kernel
-#endif
-// development ablations (results are wrong on purpose; timing only)
-#ifndef MOE_ABL
-#define MOE_ABL 0   // bit 0: no copies in the K loop, bit 1: no barrier, bit 2: copies re-read K step 0, bit 3: no FMAs, bit 4: weight copies only, bit 5: activation copies only
-#endif
-template <int XW> struct Sched {
-  static constexpr int first(int j) {
-    constexpr int n = Cfg<XW>::VM_PER_STEP, g = Cfg<XW>::XF;
-    constexpr int num = XW == 2 ? MOE_SCHED2 : MOE_SCHED1;
-    constexpr int h = (g * num) / 4 > 0 ? (g * num) / 4 : 1;   // groups that carry copies
-    if (j >= g) return n;
-    if (j <= 0) return 0;
-    if (num == 0) return n;
-    return j >= h ? n : (n * j) / h;
-  }
-};
-
 // epilogue staging tile: 128-byte rows, chunk c of row r at position c ^ (r & 7)
 __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chunk ^ (row & 7)) << 4); }
 
-template <int MODE, int XW>
-__global__ __launch_bounds__(NT, Cfg<XW>::WG_PER_CU) void grouped_gemm_kernel(
-    const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
-    const uint8_t* __restrict__ w0, const float* __restrict__ sw0,   // gate (GATEUP) or down (DOWN)
-    const uint8_t* __restrict__ w1, const float* __restrict__ sw1,   // up (GATEUP only)
-    const TileHeader* __restrict__ hdr, const TileEntry* __restrict__ tiles,
-    int K, int N,                                                    // contraction length; weight rows per matrix
-    void* __restrict__ out, float* __restrict__ out_scale) {
-  using C = Cfg<XW>;
-  constexpr int BM = C::BM, XF = C::XF, HALF = BM / 2;
-  extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-
-  // deal contiguous item ranges to the 8 XCDs (workgroup ids are issued round-robin over XCDs)
-  // work items = (row tile, column block) pairs in [expert][column block][row tile] order
-  const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
-  const int n_items = hdr->n_tiles * ncb;
-  const int per_xcd = (n_items + 7) >> 3;
-  const int slot = blockIdx.x >> 3;
-  const int item_id = (blockIdx.x & 7) * per_xcd + slot;
-  if (slot >= per_xcd || item_id >= n_items) return;
-  struct { int expert, row_start, row_count, col_block; } item;
-  {
-    const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
-    const int nt = moe_tile_count(te.rows, BM);
-    const int local = item_id - te.first_tile * ncb;
-    item.col_block = nt == 1 ? local : local / nt;
-    const int rt = local - item.col_block * nt;
-    item.expert = te.expert;
-    int t0, tn;
-    moe_tile_span(te.rows, BM, nt, rt, t0, tn);
-    item.row_start = te.row_start + t0;
-    item.row_count = tn;
-  }
-
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wi = wave & 3, xj = wave >> 2;
-  const int fr = lane & 15, fq = lane >> 4;
-  const int KB = K / BK;
-  const int e = item.expert;
-  const int wrow0 = MODE == MODE_GATEUP ? item.col_block * 128 : item.col_block * 256;
-
-  // ---- copy sources.  Wave w fills 1 KB row groups [4w, 4w+4) of the weight tile, [X_DMA w, +X_DMA) of the
-  // activation tile and BM/8 scale slots.
-  const int drow = lane >> 3, dchunk = lane & 7;
-  // the weight rows of one wave all come from one matrix: waves 0-3 copy gate rows, 4-7 up rows
-  const uint8_t* wmat = (MODE == MODE_GATEUP && wave >= 4 ? w1 : w0) + (size_t)e * N * K;   // uniform
-  // Row group i of the wave holds tile rows 32 wave + 8 i + drow: consecutive groups are 8 weight rows apart (a
-  // uniform stride, added to the scalar base when the copy is issued) and their swizzled 16-byte piece alternates
-  // between two values, so two lane offsets serve all four groups.  A wave whose 32 rows lie past the matrix (the
-  // upper half of a last, half-filled column block) reads the last 32 rows instead; nothing of what it contributes
-  // is stored.
-  unsigned woff[2];
-  {
-    int grow = MODE == MODE_GATEUP ? wrow0 + ((wave * 32) & 127) : wrow0 + wave * 32;
-    if (MODE == MODE_DOWN && grow >= N) grow = N - 32;
-    const int piece = dchunk ^ (drow >> 1);
-    woff[0] = (unsigned)(grow + drow) * (unsigned)K + piece * 16;        // < N*K <= 4 GB (checked by the launcher)
-    woff[1] = (unsigned)(grow + drow) * (unsigned)K + (piece ^ 4) * 16;
-  }
-  unsigned xoff[C::X_DMA];
-#pragma unroll
-  for (int i = 0; i < C::X_DMA; ++i) {
-    const int r = (i * NWAVES + wave) * 8 + drow;              // row within the activation tile (groups dealt round-robin)
-    const int piece = dchunk ^ ((r >> 1) & 7);
-    int g = item.row_start + min(r, item.row_count - 1);
-    if (row_ids) g = row_ids[g];
-    xoff[i] = (unsigned)g * (unsigned)K + piece * 16;          // < rows*K <= 4 GB (checked by the launcher)
-  }
-  // 16-row fragment 2j + h of the tile belongs to wave set h (its j-th), so a short tile still splits evenly between
-  // the sets.  Scale slot HALF h + fr * XF + j holds the scale of tile row 16 (2j + h) + fr: a lane reads its XF
-  // scales as XF * 4 contiguous bytes.  Wave w copies slots [BM/8 w, +BM/8).
-  unsigned soff;
-  {
-    const int p = wave * (BM / 8) + (lane & (BM / 8 - 1));
-    const int q = p % HALF;
-    const int r = 16 * (2 * (q % XF) + p / HALF) + q / XF;
-    int g = item.row_start + min(r, item.row_count - 1);
-    if (row_ids) g = row_ids[g];
-    soff = (unsigned)g * (unsigned)KB * 4u;
-  }
-  // With XSKIP, activation row groups that lie wholly past the item's last row are not copied (their LDS rows
-  // keep stale bytes; whatever the matrix cores make of them lands in rows the epilogue never stores).  Row group g
-  // (8 rows) belongs to wave g % 8, so the groups of a short tile spread over all the waves and a wave's valid
-  // groups are a prefix of its X_DMA groups.
-  const int nxv = C::XSKIP ? min(C::X_DMA, max(0, (((item.row_count + 7) >> 3) - wave + NWAVES - 1) / NWAVES)) : C::X_DMA;
-  // copy operation i (0 <= i < VM_PER_STEP) of K step kb
-  const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);   // LDS address of the ring
-  auto issue_op = [&](int kb, int i) {
-    const unsigned st = lds0 + (unsigned)(kb % C::NSTAGE) * C::STAGE_BYTES;
-    if (i < 4) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (wave * 4 + i) * 1024u);
-    else if (i < 4 + C::X_DMA) {
-      if (!C::XSKIP || i - 4 < nxv)
-        dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + ((i - 4) * NWAVES + wave) * 1024u);
-    }
-    else if (lane < BM / 8) dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4u);
-  };
-  auto issue = [&](int kb) {
-#pragma unroll
-    for (int i = 0; i < C::VM_PER_STEP; ++i) issue_op(kb, i);
-  };
-  // start the pipeline before anything else waits on memory
-  issue(0);
-  if (C::PRE > 1 && KB > 1) issue(1);
-
-  // Weight block scales of this work item go to LDS once: [0][kb] = gate (or the first 128 down rows), [1][kb] =
-  // up (or the second 128 down rows).  Scalar loads inside the K loop would force every LDS wait to
-  // lgkmcnt(0) (they share that counter and return out of order).
-  float* wscale = (float*)(lds + C::WSCALE_OFF);
-  for (int i = tid; i < 2 * KB; i += NT) {
-    const int h = i >= KB, kk = h ? i - KB : i;
-    float v;
-    if (MODE == MODE_GATEUP) v = (h ? sw1 : sw0)[((size_t)e * (N / 128) + item.col_block) * KB + kk];
-    else v = sw0[((size_t)e * (N / 128) + min(item.col_block * 2 + h, N / 128 - 1)) * KB + kk];
-    wscale[h * MAX_KB + kk] = v;
-  }
-  const float* ws0 = wscale + (MODE == MODE_GATEUP ? 0 : (wi >> 1) * MAX_KB);
-  const float* ws1 = wscale + MAX_KB;   // GATEUP only
-  __syncthreads();   // (the compiler waits here for the scale loads, and with them for the copies issued above)
-
-  const int lane_off0 = fr * BK + ((fq ^ (fr >> 1)) << 4);         // K bytes [16 fq, +16)
-  const int lane_off1 = fr * BK + (((fq + 4) ^ (fr >> 1)) << 4);   // K bytes [64 + 16 fq, +16)
-  int wfrag_off[4];                                                // byte offset of each weight fragment in the stage
-#pragma unroll
-  for (int f = 0; f < 4; ++f)
-    wfrag_off[f] = (MODE == MODE_GATEUP ? ((f >> 1) * 128 + wi * 32 + (f & 1) * 16) : (wi * 64 + f * 16)) * BK;
-  // activation fragments past the item's last row are never multiplied (uniform per wave)
-  const int jmax = (((item.row_count + 15) >> 4) + 1 - xj) >> 1;
-
-  v4f acc[4][XF];
-#pragma unroll
-  for (int f = 0; f < 4; ++f)
-#pragma unroll
-    for (int j = 0; j < XF; ++j) acc[f][j] = (v4f){0.f, 0.f, 0.f, 0.f};
-
-  auto read_frag = [&](const uint8_t* base) {
-    const v4i lo = *(const v4i*)(base + lane_off0);
-    const v4i hi = *(const v4i*)(base + lane_off1);
-    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-  };
-
-  // One K step = XF MFMA groups (one activation fragment against the wave's four weight fragments).  The two
-  // waves of a SIMD belong to different wave sets (xj = 0 / 1); set 1 runs ROT groups behind set 0, carrying the
-  // last ROT activation fragments of a step in registers across the barrier, so that after a barrier one wave of
-  // each SIMD still has matrix work in registers while the other waits for its first fragments from LDS.
-  auto run = [&](auto rot_c, auto full_c) {
-    constexpr int ROT = decltype(rot_c)::value;
-    constexpr bool FULL = decltype(full_c)::value;
-    constexpr int NG = XF - ROT;          // groups of the current step done before the next barrier
-    constexpr int XA = XW == 1 ? 2 : 1;   // activation fragments are read XA groups ahead
-    constexpr int NH = ROT > 0 ? ROT : 1;
-    v8i wf[4], held[NH];
-    float hc0[NH], hc1[NH];
-    v4f p[2][4];
-    auto mm = [&](int pp, const v8i& x) {
-#pragma unroll
-      for (int f = 0; f < 4; ++f)
-        p[pp][f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], x, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
-    };
-    auto fm = [&](int pp, int jj, float c0, float c1) {
-#pragma unroll
-      for (int f = 0; f < 4; ++f) acc[f][jj] += p[pp][f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
-    };
-    auto late = [&](bool more, int kb_next) {   // groups NG .. XF-1 of the previous step; the last FMA is left to the caller
-#pragma unroll
-      for (int i = 0; i < ROT; ++i) {
-        const int j = NG + i;
-        if (FULL || j < jmax) mm(i & 1, held[i]);
-        if (more) {
-#pragma unroll
-          for (int o = Sched<XW>::first(i); o < Sched<XW>::first(i + 1); ++o) issue_op(kb_next, o);
-        }
-        if (i > 0 && (FULL || j - 1 < jmax)) fm((i - 1) & 1, j - 1, hc0[i - 1], hc1[i - 1]);
-      }
-    };
-    for (int kb = 0; kb < KB; ++kb) {
-      // stage kb has landed once only the younger steps' copies are outstanding
-      if (C::PRE > 1 && kb + 1 < KB) wait_vm<C::VM_PER_STEP>();
-      else wait_vm<0>();
-      if (ROT > 0) wait_lgkm0();      // this wave's reads of stage kb-1 are done before anyone overwrites it
-      __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; stage (kb-1) % NSTAGE is free again
-      const bool more = kb + C::PRE < KB;   // uniform
-      if (ROT > 0) {
-        if (kb > 0) late(more, kb + C::PRE);
-        else if (more) {
-#pragma unroll
-          for (int o = 0; o < Sched<XW>::first(ROT); ++o) issue_op(kb + C::PRE, o);
-        }
-      }
-      const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
-      const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
-      const uint8_t* xt = st + C::STAGE_X_OFF + xj * 16 * BK;
-#pragma unroll
-      for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
-      float sxv[XF];
-#pragma unroll
-      for (int j = 0; j < XF; j += 4) {
-        if constexpr (XF >= 4) {
-          const v4f a = *(const v4f*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + j * 4);
-          sxv[j] = a[0]; sxv[j + 1] = a[1]; sxv[j + 2] = a[2]; sxv[j + 3] = a[3];
-        } else {
-#pragma unroll
-          for (int q = 0; q < XF; ++q) sxv[q] = *(const float*)(st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4 + q * 4);
-        }
-      }
-      v8i xf[XA + 1];
-#pragma unroll
-      for (int j = 0; j < XA; ++j) xf[j] = read_frag(xt + j * 32 * BK);
-      if constexpr (ROT > 0) {
-        if (kb > 0 && (FULL || XF - 1 < jmax)) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
-      }
-#pragma unroll
-      for (int j = 0; j <= NG; ++j) {
-        if (j + XA < NG) xf[(j + XA) % (XA + 1)] = read_frag(xt + (j + XA) * 32 * BK);
-        if (j < NG && (FULL || j < jmax)) mm(j & 1, xf[j % (XA + 1)]);
-        // the copies for step kb + PRE are spread over the MFMA groups: issued in one burst they hold every wave
-        // at the memory pipeline's front door while the matrix cores idle
-        if (j < NG && more) {
-#pragma unroll
-          for (int o = Sched<XW>::first(ROT + j); o < Sched<XW>::first(ROT + j + 1); ++o) issue_op(kb + C::PRE, o);
-        }
-        if (ROT > 0 && j == 0) {
-#pragma unroll
-          for (int i = 0; i < ROT; ++i) {
-            held[i] = read_frag(xt + (NG + i) * 32 * BK);
-            hc0[i] = sxv[NG + i] * s0;
-            hc1[i] = sxv[NG + i] * s1;
-          }
-        }
-        if (j > 0 && (FULL || j - 1 < jmax)) fm((j - 1) & 1, j - 1, sxv[j - 1] * s0, sxv[j - 1] * s1);
-      }
-    }
-    if constexpr (ROT > 0) {
-      late(false, 0);
-      if (FULL || XF - 1 < jmax) fm((ROT - 1) & 1, XF - 1, hc0[ROT - 1], hc1[ROT - 1]);
-    }
-  };
-  // one uniform branch per work item: the common full tile runs a branch-free schedule
-  // (at BM = 256 two copies of the schedule do not fit the register file next to 128 accumulators)
-  constexpr int ROT = C::ROT;
-  const bool full = XW == 1 && jmax == XF;
-  if (ROT == 0 || xj == 0) {
-    if (full) run(std::integral_constant<int, 0>{}, std::true_type{});
-    else run(std::integral_constant<int, 0>{}, std::false_type{});
-  } else {
-    if (full) run(std::integral_constant<int, ROT>{}, std::true_type{});
-    else run(std::integral_constant<int, ROT>{}, std::false_type{});
-  }
-  __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
-
-  // ---- epilogue.  Lane holds, for fragment (f, j): tile row (2j + xj)*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
-  if (MODE == MODE_GATEUP) {
-    float* amax_s = (float*)lds;                       // [4 weight-wave groups][BM rows]
-    uint8_t* tile = lds + 4 * BM * sizeof(float);      // [BM rows][128 B], swizzled
-#pragma unroll
-    for (int j = 0; j < XF; ++j) {
-      float m = 0.f;
-#pragma unroll
-      for (int f = 0; f < 2; ++f)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float g = acc[f][j][r], u = acc[f + 2][j][r];
-          float h = g / (1.0f + __expf(-g)) * u;
-          acc[f][j][r] = h;
-          m = fmaxf(m, fabsf(h));
-        }
-      m = fmaxf(m, __shfl_xor(m, 16, MOE_WAVE));
-      m = fmaxf(m, __shfl_xor(m, 32, MOE_WAVE));
-      if (fq == 0) amax_s[wi * BM + (2 * j + xj) * 16 + fr] = m;
-    }
-    __syncthreads();
-    const int I = N;
-    uint8_t* hq = (uint8_t*)out;
-#pragma unroll
-    for (int j = 0; j < XF; ++j) {
-      const int xr = (2 * j + xj) * 16 + fr;
-      float m = fmaxf(fmaxf(amax_s[xr], amax_s[BM + xr]), fmaxf(amax_s[2 * BM + xr], amax_s[3 * BM + xr]));
-      float scale, scale_inv;
-      fp8_scales(m, scale, scale_inv);
-#pragma unroll
-      for (int f = 0; f < 2; ++f) {
-        unsigned q = pack4_e4m3(acc[f][j][0] * scale, acc[f][j][1] * scale, acc[f][j][2] * scale, acc[f][j][3] * scale);
-        const int col = wi * 32 + f * 16 + fq * 4;  // byte column within the 128-wide slab
-        *(unsigned*)(tile + swz(xr, col >> 4) + (col & 15)) = q;
-      }
-      if (wi == 0 && fq == 0 && xr < item.row_count)
-        out_scale[(size_t)(item.row_start + xr) * (I / 128) + item.col_block] = scale_inv;
-    }
-    __syncthreads();
-    const int ld_chunk = tid & 7, ld_row = tid >> 3;   // 64 rows per pass
-#pragma unroll
-    for (int i = 0; i < (BM + 63) / 64; ++i) {
-      const int r = ld_row + 64 * i;
-      if (r < item.row_count) {
-        v4i v = *(const v4i*)(tile + swz(r, ld_chunk));
-        *(v4i*)(hq + (size_t)(item.row_start + r) * I + item.col_block * 128 + ld_chunk * 16) = v;
-      }
-    }
-  } else {
-    // bf16 tile [BM rows][256 cols] = 512 B per row, 32 chunks of 16 B, swizzled with (row & 7)
-    uint8_t* tile = lds;
-#pragma unroll
-    for (int j = 0; j < XF; ++j) {
-      const int xr = (2 * j + xj) * 16 + fr;
-#pragma unroll
-      for (int f = 0; f < 4; ++f) {
-        const int col = wi * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
-        uint2 v;
-        v.x = (unsigned)f32_to_bf16(acc[f][j][0]) | ((unsigned)f32_to_bf16(acc[f][j][1]) << 16);
-        v.y = (unsigned)f32_to_bf16(acc[f][j][2]) | ((unsigned)f32_to_bf16(acc[f][j][3]) << 16);
-        const int chunk = col >> 3;  // 8 bf16 per 16-byte chunk
-        *(uint2*)(tile + xr * 512 + ((chunk ^ (xr & 7)) << 4) + (col & 7) * 2) = v;
-      }
-    }
-    __syncthreads();
-    bf16_t* y = (bf16_t*)out;
-    const int c32 = tid & 31, r16 = tid >> 5;          // 16 rows per pass
-    const int ncols = min(256, N - wrow0);
-#pragma unroll
-    for (int i = 0; i < BM / 16; ++i) {
-      const int r = r16 + 16 * i;
-      if (r < item.row_count && c32 * 8 < ncols) {
-        v4i v = *(const v4i*)(tile + r * 512 + ((c32 ^ (r & 7)) << 4));
-        *(v4i*)(y + (size_t)(item.row_start + r) * N + wrow0 + c32 * 8) = v;
-      }
-    }
-  }
-}
-
-// ---- tile-class kernel ---------------------------------------------------------------------------------------
-//
-// One launch, row tiles of every height.  A work item's row tile (at most 256 rows, equal-height cuts of its
+// One launch, row tiles of every height.  A work item's row tile (at most 256 rows, near-equal cuts of its
 // expert) is served by the smallest of eight compiled tile classes that holds it -- 32 XF rows, XF = 1 .. 8 MFMA
 // groups per wave and K step -- each a branch-free, fully unrolled K loop of its own with its own LDS ring: the
 // short classes have short activation tiles and use the room for more stages (160 rows and more: two stages,
@@ -602,9 +196,6 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);
   auto issue_op = [&](int kb, int i) {
     const unsigned st = lds0 + (unsigned)(kb % C::NSTAGE) * C::STAGE_BYTES;
-    if ((MOE_ABL & 16) && i >= 4) return;
-    if ((MOE_ABL & 32) && i < 4) return;
-    if (MOE_ABL & 4) kb = 0;
     if (i < 4) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (wave * 4 + i) * 1024u);
     else if (i < 4 + C::X_OPS) {
       int grp = (i - 4) * NWAVES + wave;
@@ -652,13 +243,13 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   v4f p[4];
   float pc0 = 0.f, pc1 = 0.f;   // scales of the group whose FMAs are pending
   auto fm = [&](int f, int jj, float c0, float c1) {
-    if (!(MOE_ABL & 8)) acc[f][jj] += p[f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
+    acc[f][jj] += p[f] * ((MODE == MODE_GATEUP && f >= 2) ? c1 : c0);
   };
   auto mm = [&](int f, const v8i& x) {
     p[f] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[f], x, (v4f){0.f, 0.f, 0.f, 0.f}, 0, 0, 0, 0, 0, 0);
   };
   auto fence = [&]() {
-    if (MOE_FENCE) __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_sched_barrier(0);
   };
   // The two waves of a SIMD belong to different wave sets (xj = 0 / 1).  Set 1 runs ROT groups behind set 0: it
   // carries the last ROT activation fragments of a step (and their scales) in registers across the barrier and
@@ -682,7 +273,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
         else wait_vm<0>();
       }
       if (ROT > 0) wait_lgkm0();      // this wave's reads of stage kb - 1 are done before anyone overwrites it
-      if (!(MOE_ABL & 2)) __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; every wave is done with stage kb - 1
+      __builtin_amdgcn_s_barrier();   // stage kb is complete for every wave; every wave is done with stage kb - 1
       if constexpr (ROT > 0) {        // groups NG .. XF-1 of the previous step: held fragments, the previous weights
         if (!FIRST) {
 #pragma unroll
@@ -694,13 +285,13 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
             }
             pc0 = hc0[i];
             pc1 = hc1[i];
-            if (COPY && !(MOE_ABL & 1)) {
+            if (COPY) {
 #pragma unroll
               for (int o = C::first(i); o < C::first(i + 1); ++o) issue_op(kb + C::PRE, o);
             }
             fence();
           }
-        } else if (COPY && !(MOE_ABL & 1)) {
+        } else if (COPY) {
 #pragma unroll
           for (int o = 0; o < C::first(ROT); ++o) issue_op(kb + C::PRE, o);
         }
@@ -708,12 +299,11 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
       const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
       const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
       const uint8_t* xt = st + C::STAGE_X_OFF + xj * 16 * BK;
-      // finish the previous step's last group first: its FMAs need the last MFMAs' results, and those MFMAs
-      // are still reading the weight fragments that the reads below overwrite
-      if (!FIRST) {
-#pragma unroll
-        for (int f = 0; f < 4; ++f) fm(f, XF - 1, pc0, pc1);
-      }
+      // Every wave of a wave set asks LDS for its first fragments at this moment: the reads come back in issue
+      // order, so the first MFMA's operands (activation fragment 0, weight fragment 0) are asked for first and the
+      // scales last; the FMAs that finish the previous step's last group run while the reads travel.
+      v8i xf[2];
+      xf[0] = read_frag(xt);
 #pragma unroll
       for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
       float sxv[XF];
@@ -736,8 +326,10 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
           for (int j = 0; j < XF; ++j) sxv[j] = *(const float*)(sp + j * 4);
         }
       }
-      v8i xf[2];
-      xf[0] = read_frag(xt);
+      if (!FIRST) {
+#pragma unroll
+        for (int f = 0; f < 4; ++f) fm(f, XF - 1, pc0, pc1);
+      }
       fence();
 #pragma unroll
       for (int j = 0; j < NG; ++j) {
@@ -757,7 +349,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
         }
         pc0 = sxv[j] * s0;
         pc1 = sxv[j] * s1;
-        if (COPY && !(MOE_ABL & 1)) {
+        if (COPY) {
 #pragma unroll
           for (int o = C::first(ROT + j); o < C::first(ROT + j + 1); ++o) issue_op(kb + C::PRE, o);
         }
@@ -787,9 +379,9 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
 #pragma unroll
     for (int f = 0; f < 4; ++f) fm(f, XF - 1, pc0, pc1);
   };
-  constexpr int ROTC = XF >= 3 ? MOE_ROTC : XF - 1;   // (fewer groups than that: what there is)
-  if (ROTC == 0 || xj == 0) run(std::integral_constant<int, 0>{});
-  else run(std::integral_constant<int, ROTC>{});
+  constexpr int ROT1 = XF > ROTC ? ROTC : XF - 1;   // (fewer groups than that: what there is)
+  if (ROT1 == 0 || xj == 0) run(std::integral_constant<int, 0>{});
+  else run(std::integral_constant<int, ROT1>{});
   __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
 
   // ---- epilogue.  Lane holds, for fragment (f, j): tile row (2j + xj)*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
@@ -872,7 +464,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
 }
 
 template <int MODE>
-__global__ __launch_bounds__(NT, 1) void grouped_gemm_classes_kernel(
+__global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0, const uint8_t* __restrict__ w1,
     const float* __restrict__ sw1, const TileHeader* __restrict__ hdr, const TileEntry* __restrict__ tiles, int K,
@@ -889,22 +481,18 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_classes_kernel(
   Item item;
   {
     const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
-    const int nt = moe_tile_count(te.rows, 256);
+    const int nt = moe_tile_count(te.rows);
     const int local = item_id - te.first_tile * ncb;
     item.col_block = nt == 1 ? local : local / nt;
     const int rt = local - item.col_block * nt;
     item.expert = te.expert;
     int t0, tn;
-    moe_tile_span(te.rows, 256, nt, rt, t0, tn);
+    moe_tile_span(te.rows, nt, rt, t0, tn);
     item.row_start = te.row_start + t0;
     item.row_count = tn;
   }
   const int rows = __builtin_amdgcn_readfirstlane(item.row_count);
 #define MOE_ITEM(XF) item_body<MODE, XF>(item, lds, xq, sx, row_ids, w0, sw0, w1, sw1, K, N, out, out_scale)
-#ifdef MOE_ONLY_XF
-  (void)rows;
-  MOE_ITEM(MOE_ONLY_XF);
-#else
   switch ((rows + 31) >> 5) {
     case 8: MOE_ITEM(8); break;
     case 7: MOE_ITEM(7); break;
@@ -915,67 +503,15 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_classes_kernel(
     case 2: MOE_ITEM(2); break;
     default: MOE_ITEM(1); break;
   }
-#endif
 #undef MOE_ITEM
 }
-
 int col_blocks(int mode, int N) { return mode == MODE_GATEUP ? N / 128 : (N + 255) / 256; }
 
-int max_tiles_for(int R, int E, int bm) { return (int)((long long)(R + bm - 1) / bm + (E < R ? E : R)); }
+int max_tiles_for(int R, int E) { return (int)((long long)(R + 255) / 256 + (E < R ? E : R)); }
 
-TileList tile_list(void* ws, int R, int E, int bm) {
-  return TileList{max_tiles_for(R, E, bm), (TileHeader*)ws, (TileEntry*)((char*)ws + sizeof(TileHeader))};
+TileList tile_list(void* ws, int R, int E) {
+  return TileList{max_tiles_for(R, E), (TileHeader*)ws, (TileEntry*)((char*)ws + sizeof(TileHeader))};
 }
-
-template <int MODE, int XW>
-int launch_cfg(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
-               const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
-               void* out, float* out_scale, void* ws, bool list_built, hipStream_t s) {
-  using C = Cfg<XW>;
-  const TileList l = tile_list(ws, R, E, C::BM);
-  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, C::BM, l);
-  static std::atomic<unsigned long long> lds_raised{0};
-  if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE, XW>, C::LDS_BYTES, lds_raised)) return rc;
-  const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
-  MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
-  const int grid = (int)((max_items + 7) / 8) * 8;
-  hipLaunchKernelGGL((grouped_gemm_kernel<MODE, XW>), dim3(grid), dim3(NT), C::LDS_BYTES, s, xq, sx, row_ids, w0, sw0,
-                     w1, sw1, l.hdr, l.tiles, K, N, out, out_scale);
-  return moe_check_hip(hipGetLastError(), "gemm launch");
-}
-
-template <int MODE>
-int launch_classes(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
-                   const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
-                   void* out, float* out_scale, void* ws, bool list_built, hipStream_t s) {
-  const TileList l = tile_list(ws, R, E, 256);
-  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, 256, l);
-  static std::atomic<unsigned long long> lds_raised{0};
-  if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_classes_kernel<MODE>, CLS_LDS_BYTES, lds_raised)) return rc;
-  const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
-  MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
-  const int grid = (int)((max_items + 7) / 8) * 8;
-  hipLaunchKernelGGL((grouped_gemm_classes_kernel<MODE>), dim3(grid), dim3(NT), CLS_LDS_BYTES, s, xq, sx, row_ids, w0,
-                     sw0, w1, sw1, l.hdr, l.tiles, K, N, out, out_scale);
-  return moe_check_hip(hipGetLastError(), "gemm launch");
-}
-
-// MOE_GEMM_BM=32|256 in the environment pins the kernel for experiments; default: by shape
-int forced_cfg() {
-  static int v = [] {
-    const char* e = getenv("MOE_GEMM_BM");
-    return e ? atoi(e) : 0;
-  }();
-  return v == 32 ? 0 : v == 256 ? 2 : -1;
-}
-
-// Batches of at most 16 rows per expert on average run the 32-row kernel with two workgroups per CU (one streams
-// weights while the other starts or finishes an item); everything else runs the tile-class kernel.
-int tile_config(int R, int E) {
-  if (forced_cfg() >= 0) return forced_cfg();
-  return (long long)R <= 16ll * E ? 0 : 2;
-}
-int tile_height(int cfg) { return cfg == 0 ? 32 : 256; }
 
 template <int MODE>
 int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
@@ -987,19 +523,23 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
   MOE_REQUIRE((long long)N * K <= (1ll << 32) && (long long)R * K <= (1ll << 32), MOE_ERR_BAD_SHAPE,
               "gemm: one expert matrix and the activation array must each stay within 4 GB (N=%d K=%d R=%d)", N, K, R);
   if (R == 0) return MOE_OK;
-  if (tile_config(R, E) == 0)
-    return launch_cfg<MODE, 0>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
-                               list_built, s);
-  return launch_classes<MODE>(xq, sx, row_ids, w0, sw0, w1, sw1, group_offsets, E, R, K, N, out, out_scale, ws,
-                              list_built, s);
+  const TileList l = tile_list(ws, R, E);
+  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, l);
+  static std::atomic<unsigned long long> lds_raised{0};
+  if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE>, CLS_LDS_BYTES, lds_raised)) return rc;
+  const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
+  MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
+  const int grid = (int)((max_items + 7) / 8) * 8;   // sized by the worst case; surplus workgroups exit at once
+  hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NT), CLS_LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1,
+                     sw1, l.hdr, l.tiles, K, N, out, out_scale);
+  return moe_check_hip(hipGetLastError(), "gemm launch");
 }
 
 }  // namespace
 
 extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
   (void)N_out;   // the tile list does not depend on the number of output columns
-  const int bm = tile_height(tile_config(R, E));
-  return sizeof(TileHeader) + (size_t)max_tiles_for(R, E, bm) * sizeof(TileEntry) + 256;
+  return sizeof(TileHeader) + (size_t)max_tiles_for(R, E) * sizeof(TileEntry) + 256;
 }
 
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
@@ -1082,11 +622,10 @@ extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8
 }
 
 // The tile list that the GEMM launches of (R rows, E experts) read from ws when they are told list_built = true.
-int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list, int* bm) {
-  MOE_REQUIRE(ws && list && bm, MOE_ERR_NULL, "gemm tiles: null pointer");
+int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list) {
+  MOE_REQUIRE(ws && list, MOE_ERR_NULL, "gemm tiles: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0, MOE_ERR_BAD_SHAPE, "gemm tiles: need 1 <= E <= 1024, got E=%d R=%d", E, R);
   MOE_REQUIRE(ws_bytes >= moe_gemm_workspace_bytes(R, E, 0), MOE_ERR_WORKSPACE_TOO_SMALL, "gemm tiles: workspace too small");
-  *bm = tile_height(tile_config(R, E));
-  *list = tile_list(ws, R, E, *bm);
+  *list = tile_list(ws, R, E);
   return MOE_OK;
 }

@@ -59,10 +59,10 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(const int32_t* __restric
 // one workgroup: thread e owns expert e (loop if E > blockDim)
 __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk_hist, int n_chunks, int E,
                                                     int32_t* __restrict__ group_sizes,
-                                                    int32_t* __restrict__ group_offsets, TileList tl, int bm) {
+                                                    int32_t* __restrict__ group_offsets, TileList tl) {
   __shared__ int tot[kMaxE];
   __shared__ int wave_tot[kMaxE / MOE_WAVE];
-  __shared__ int wave_tiles[kMaxE / MOE_WAVE];
+  __shared__ int tile_key[kMaxE];
   const int e = threadIdx.x;
   int total = 0;
   if (e < E) {
@@ -92,21 +92,11 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
     if (e == E - 1) group_offsets[E] = excl + total;
     for (int c = 0; c < n_chunks; ++c) chunk_hist[(size_t)c * E + e] += excl;  // absolute first position
   }
-  if (tl.tiles) {   // the grouped GEMMs' row tiles, [expert][tile] (uniform branch)
-    const int nt = e < E ? moe_tile_count(total, bm) : 0;
-    int tincl = nt;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      int o = __shfl_up(tincl, off, MOE_WAVE);
-      if (lane >= off) tincl += o;
-    }
-    if (lane == 63) wave_tiles[wv] = tincl;
-    __syncthreads();
-    int first = tincl - nt, all = 0;
-    for (int i = 0; i < kMaxE / MOE_WAVE; ++i) {
-      if (i < wv) first += wave_tiles[i];
-      all += wave_tiles[i];
-    }
+  if (tl.tiles) {   // the grouped GEMMs' row tiles, an expert's tiles side by side (uniform branch)
+    __syncthreads();   // (tot is read above by nobody else: it doubles as the helper's scratch from here on)
+    int all = 0;
+    const int nt = e < E ? moe_tile_count(total) : 0;
+    const int first = moe_tile_first(e, E, e < E ? total : 0, tot, tile_key, &all);
     for (int t = 0; t < nt; ++t)
       if (first + t < tl.max_tiles) tl.tiles[first + t] = TileEntry{e, excl, total, first};
     if (e == 0) tl.hdr->n_tiles = all < tl.max_tiles ? all : tl.max_tiles;
@@ -156,7 +146,7 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
                                                                 int32_t* __restrict__ group_offsets,
                                                                 int32_t* __restrict__ sorted_token_ids,
                                                                 int32_t* __restrict__ sort_order,
-                                                                int32_t* __restrict__ inv_perm, TileList tl, int bm) {
+                                                                int32_t* __restrict__ inv_perm, TileList tl) {
   __shared__ int hist[kMaxE];   // counts, then next free output position per expert
   __shared__ int wave_tot[kWaves];
   __shared__ int wave_tiles[kWaves];
@@ -196,7 +186,7 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
   int nt = 0, tincl = 0;
   if (tl.tiles) {   // the grouped GEMMs' row tiles, [expert][tile] (uniform branch)
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) nt += moe_tile_count(c[i], bm);   // (experts >= E count nothing)
+    for (int i = 0; i < kPer; ++i) nt += moe_tile_count(c[i]);   // (experts >= E count nothing)
     tincl = nt;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -225,7 +215,7 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
       if (e == E - 1) group_offsets[E] = run + c[i];
     }
     if (tl.tiles) {
-      const int n = moe_tile_count(c[i], bm);
+      const int n = moe_tile_count(c[i]);
       for (int t = 0; t < n; ++t)
         if (first + t < tl.max_tiles) tl.tiles[first + t] = TileEntry{e, run, c[i], first};
       first += n;
@@ -269,7 +259,7 @@ extern "C" size_t moe_permute_workspace_bytes(int M, int k, int E) {
 
 int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_sizes, int32_t* group_offsets,
                      int32_t* sorted_token_ids, int32_t* sort_order, int32_t* inv_perm, void* ws, size_t ws_bytes,
-                     TileList tiles, int bm, moe_stream_t stream) {
+                     TileList tiles, moe_stream_t stream) {
   MOE_REQUIRE((idx || M == 0) && group_sizes && group_offsets && ws, MOE_ERR_NULL, "permute: null pointer");
   MOE_REQUIRE(M >= 0 && k >= 1 && E >= 1 && E <= kMaxE, MOE_ERR_BAD_SHAPE,
               "permute: need k >= 1 and 1 <= E <= %d, got M=%d k=%d E=%d", kMaxE, M, k, E);
@@ -282,13 +272,13 @@ int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_siz
   if (n_chunks < 1) n_chunks = 1;
   if (R <= kChunk) {
     hipLaunchKernelGGL(permute_small_kernel, dim3(1), dim3(kThreads), 0, s, idx, R, E, k, group_sizes, group_offsets,
-                       sorted_token_ids, sort_order, inv_perm, tiles, bm);
+                       sorted_token_ids, sort_order, inv_perm, tiles);
     return moe_check_hip(hipGetLastError(), "permute launch");
   }
   int32_t* chunk_hist = (int32_t*)ws;
   hipLaunchKernelGGL(hist_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, chunk_hist);
   hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kMaxE), 0, s, chunk_hist, n_chunks, E, group_sizes, group_offsets,
-                     tiles, bm);
+                     tiles);
   if (R > 0 && (sorted_token_ids || sort_order || inv_perm))
     hipLaunchKernelGGL(scatter_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, k,
                        chunk_hist, sorted_token_ids, sort_order, inv_perm);
@@ -299,5 +289,5 @@ extern "C" int moe_permute(const int32_t* idx, int M, int k, int E, int32_t* gro
                            int32_t* group_offsets, int32_t* sorted_token_ids, int32_t* sort_order,
                            int32_t* inv_perm, void* ws, size_t ws_bytes, moe_stream_t stream) {
   return moe_permute_impl(idx, M, k, E, group_sizes, group_offsets, sorted_token_ids, sort_order, inv_perm, ws,
-                          ws_bytes, TileList{0, nullptr, nullptr}, 1, stream);
+                          ws_bytes, TileList{0, nullptr, nullptr}, stream);
 }

@@ -148,8 +148,8 @@ def _ragged_case(seed, E, D, I, sizes):
     (8, 512, 1024, [64] * 8),
     (3, 384, 384, [257, 0, 1]),           # D % 256 != 0: the down GEMM's last column block is half full
     (6, 2048, 768, [300, 0, 0, 129, 7, 64]),
-    (8, 256, 256, [70, 0, 1, 33, 0, 16, 0, 0]),   # <= 16 rows per expert on average: 32-row tiles, several per expert
-    (2, 256, 256, [300, 150]),                    # > 128 rows per expert on average: 256-row tiles, equal-height split
+    (8, 256, 256, [70, 0, 1, 33, 0, 16, 0, 0]),   # a few rows per expert: the 32- and 64-row tile classes, empty experts between
+    (2, 256, 256, [300, 150]),                    # two row tiles for one expert (near-equal cut), one 160-row tile for the other
 ])
 def test_grouped_gemms_vs_oracle(jg, E, D, I, sizes):
     _say("grouped_gemm", E, D, I, sizes)
