@@ -220,7 +220,7 @@ def run_ep_shard(jg, torch, steps, warmup, seed=5):
                        "touched_experts": touched, "largest_group": int(group_sizes.max()), "group_sizes": "Zipf(1.2)"},
             "roofline": {"bound": "mfma", "achieved": k_flops / k_ms / 1e9, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                          "frac": k_flops / k_ms / 1e9 / PEAK_FP8_TFLOPS, "traffic": None,
-                         "kernel": "grouped_gemm_classes_kernel<0> (gate/up + SwiGLU + h quantisation), rows in expert order",
+                         "kernel": "grouped_gemm_kernel<0> (gate/up + SwiGLU + h quantisation), rows in expert order",
                          "avg_launch_ms": k_ms, "flops_per_launch": k_flops}}
 
 
@@ -304,7 +304,7 @@ def main():
         traffic, traffic_src = measured_traffic(args.workload) if args.bias_std == 0.1 else (None, None)
         roof = {"bound": "mfma", "achieved": gk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                 "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
-                "kernel": "grouped_gemm_classes_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
+                "kernel": "grouped_gemm_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
                 "algorithmic_bytes_per_launch": gk["bytes_per_launch"],
                 "avg_launch_ms": gk["avg_launch_ms"], "flops_per_launch": gk["flops_per_launch"]}
     line = {
@@ -328,7 +328,7 @@ def main():
                                        "traffic": measured_traffic("deepseek_v3_decode")[0],
                                        "traffic_source": measured_traffic("deepseek_v3_decode")[1],
                                        "algorithmic_bytes_per_launch": dk["bytes_per_launch"],
-                                       "kernel": "grouped_gemm_kernel<0, 0>, routed launch (gate/up + SwiGLU + h quantisation)",
+                                       "kernel": "grouped_gemm_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
                                        "avg_launch_ms": dk["avg_launch_ms"]}}
     if qwen3:
         qk = qwen3["gateup_kernel"]
@@ -338,7 +338,7 @@ def main():
                                                 "touched_experts": qwen3["touched_experts"]},
                                      "roofline": {"bound": "mfma", "achieved": qk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                                                   "frac": qk["tflops"] / PEAK_FP8_TFLOPS, "traffic": None,
-                                                  "kernel": "grouped_gemm_classes_kernel<0>, routed launch", "avg_launch_ms": qk["avg_launch_ms"],
+                                                  "kernel": "grouped_gemm_kernel<0>, routed launch", "avg_launch_ms": qk["avg_launch_ms"],
                                                   "flops_per_launch": qk["flops_per_launch"]}}
     if ep_shard:
         line["ep_shard_skewed"] = ep_shard
