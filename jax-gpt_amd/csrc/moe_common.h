@@ -155,6 +155,14 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {  // round-to-nearest-ev
   return (bf16_t)(u >> 16);
 }
 
+// two f32 -> two bf16 (RNE) in one dword, low half first: the hardware's packed conversion
+__device__ __forceinline__ unsigned pack2_bf16(float lo, float hi) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+  const bf16x2_hw b = __builtin_convertvector((f32x2){lo, hi}, bf16x2_hw);
+  return __builtin_bit_cast(unsigned, b);
+}
+
 // scale = 448/amax (1 when the group is all zero); both quotients are IEEE-rounded
 __device__ __forceinline__ void fp8_scales(float amax, float& scale, float& scale_inv) {
   scale = amax > 0.f ? __fdiv_rn(MOE_FP8_MAX, amax) : 1.0f;

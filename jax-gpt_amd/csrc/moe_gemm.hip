@@ -396,7 +396,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float g = acc[f][j][r], u = acc[f + 2][j][r];
-          float h = g / (1.0f + __expf(-g)) * u;
+          float h = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;   // (reciprocal to 1 ulp: far inside the fp8 step)
           acc[f][j][r] = h;
           m = fmaxf(m, fabsf(h));
         }
@@ -415,7 +415,11 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
       fp8_scales(m, scale, scale_inv);
 #pragma unroll
       for (int f = 0; f < 2; ++f) {
-        unsigned q = pack4_e4m3(acc[f][j][0] * scale, acc[f][j][1] * scale, acc[f][j][2] * scale, acc[f][j][3] * scale);
+        int q = 0;   // (|h| <= amax, so the products stay within a rounding of +-448: one median clamps them)
+        q = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(acc[f][j][0] * scale, -MOE_FP8_MAX, MOE_FP8_MAX),
+                                            __builtin_amdgcn_fmed3f(acc[f][j][1] * scale, -MOE_FP8_MAX, MOE_FP8_MAX), q, false);
+        q = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(acc[f][j][2] * scale, -MOE_FP8_MAX, MOE_FP8_MAX),
+                                            __builtin_amdgcn_fmed3f(acc[f][j][3] * scale, -MOE_FP8_MAX, MOE_FP8_MAX), q, true);
         const int col = wi * 32 + f * 16 + fq * 4;  // byte column within the 128-wide slab
         *(unsigned*)(tile + swz(xr, col >> 4) + (col & 15)) = q;
       }
@@ -442,8 +446,8 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
       for (int f = 0; f < 4; ++f) {
         const int col = wi * 64 + f * 16 + fq * 4;  // output column within the 256-wide slab
         uint2 v;
-        v.x = (unsigned)f32_to_bf16(acc[f][j][0]) | ((unsigned)f32_to_bf16(acc[f][j][1]) << 16);
-        v.y = (unsigned)f32_to_bf16(acc[f][j][2]) | ((unsigned)f32_to_bf16(acc[f][j][3]) << 16);
+        v.x = pack2_bf16(acc[f][j][0], acc[f][j][1]);
+        v.y = pack2_bf16(acc[f][j][2], acc[f][j][3]);
         const int chunk = col >> 3;  // 8 bf16 per 16-byte chunk
         *(uint2*)(tile + xr * 512 + ((chunk ^ (xr & 7)) << 4) + (col & 7) * 2) = v;
       }

@@ -64,12 +64,16 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
   __shared__ int wave_tot[kMaxE / MOE_WAVE];
   __shared__ int tile_key[kMaxE];
   const int e = threadIdx.x;
+  // (the chunk loops read in batches of independent loads: one load at a time would pay a memory round trip per chunk)
+  constexpr int kBatch = 8;
   int total = 0;
   if (e < E) {
-    for (int c = 0; c < n_chunks; ++c) {  // exclusive scan down the chunks, in place
-      int v = chunk_hist[(size_t)c * E + e];
-      chunk_hist[(size_t)c * E + e] = total;
-      total += v;
+    for (int c0 = 0; c0 < n_chunks; c0 += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v[i] = c0 + i < n_chunks ? chunk_hist[(size_t)(c0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) total += v[i];
     }
     group_sizes[e] = total;
   }
@@ -90,7 +94,18 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
   if (e < E) {
     group_offsets[e] = excl;
     if (e == E - 1) group_offsets[E] = excl + total;
-    for (int c = 0; c < n_chunks; ++c) chunk_hist[(size_t)c * E + e] += excl;  // absolute first position
+    int run = excl;   // counts -> absolute first position of the expert's rows within each chunk, in place
+    for (int c0 = 0; c0 < n_chunks; c0 += kBatch) {
+      int v[kBatch];
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i) v[i] = c0 + i < n_chunks ? chunk_hist[(size_t)(c0 + i) * E + e] : 0;
+#pragma unroll
+      for (int i = 0; i < kBatch; ++i)
+        if (c0 + i < n_chunks) {
+          chunk_hist[(size_t)(c0 + i) * E + e] = run;
+          run += v[i];
+        }
+    }
   }
   if (tl.tiles) {   // the grouped GEMMs' row tiles, an expert's tiles side by side (uniform branch)
     __syncthreads();   // (tot is read above by nobody else: it doubles as the helper's scratch from here on)
