@@ -41,7 +41,18 @@ inline int moe_raise_lds_limit(const void* kernel, int bytes, std::atomic<unsign
 struct TileHeader {
   int n_tiles;
   int pad[3];
+  // Where the work of XCD k begins, as a tile position with 20 fraction bits (xcd_q[0] = 0, xcd_q[8] = n_tiles << 20);
+  // a GEMM with ncb column blocks per row tile gives XCD k the items [xcd_q[k] * ncb >> 20, xcd_q[k + 1] * ncb >> 20).
+  long long xcd_q[9];
+  long long pad2;
 };
+constexpr int kTileQBits = 20;
+// The grouped GEMM launches ceil(max_tiles * ncb / 8) + 2 workgroups per XCD: a split whose largest share stays
+// within max_tiles / 8 tiles fits whatever ncb is (max_tiles is a worst case over all group sizes, so a real list
+// is usually a good deal shorter and its shares fit with room to spare).
+__host__ __device__ inline long long moe_xcd_share_cap_q(int max_tiles) {
+  return ((long long)max_tiles << kTileQBits) >> 3;
+}
 struct TileEntry {
   int expert, row_start, rows, first_tile;
 };
@@ -76,8 +87,20 @@ __host__ __device__ inline void moe_tile_span(int rows, int nt, int t, int& star
 // experts largest first.
 // Called by every thread of a workgroup with at least E threads; thread e owns expert e (rows = 0 for e >= E);
 // lds_rows and lds_key are int[blockDim.x] arrays in LDS.  Returns the index of expert e's first tile and, in
-// *total_tiles, the length of the list.
-__device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int* lds_key, int* total_tiles) {
+// *total_tiles, the length of the list, and writes the list header.
+//
+// The header's XCD shares are cut by cost, not by count: a row tile of u 32-row units costs about 8 + u (measured:
+// 63 us for a 32-row tile of the gate/up GEMM against 112 us for a 256-row one, and the same ratio for the down
+// GEMM), and equal counts left the XCD with the tallest tiles some 3 % more work than the average.  All tiles of an
+// expert cost alike, so a cut inside an expert sits at the same fraction of its items as of its cost.
+__device__ inline int moe_tile_cost(int rows) { return 8 * moe_tile_count(rows) + ((rows + 31) >> 5); }   // (< 2^31 for 2^32 / 128 rows)
+__device__ inline void moe_tile_even_shares(TileHeader* hdr, int n_tiles) {   // one thread
+  hdr->n_tiles = n_tiles;
+  for (int k = 0; k <= 8; ++k) hdr->xcd_q[k] = (((long long)n_tiles << kTileQBits) * k) >> 3;
+}
+__device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int* lds_key, int* total_tiles,
+                                     TileHeader* hdr, int max_tiles) {
+  __shared__ long long cut_q[9];
   lds_rows[e] = e < E ? rows : 0;
   __syncthreads();
   int key = e;
@@ -94,13 +117,43 @@ __device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int*
   lds_key[e] = key;
   __syncthreads();
   int first = 0, total = 0;
+  int cost_before = 0, cost_all = 0;
 #pragma unroll 8
   for (int o = 0; o < E; ++o) {
     const int t = moe_tile_count(lds_rows[o]);
+    const int c = 8 * t + ((lds_rows[o] + 31) >> 5);
+    const bool before = lds_key[o] < key;
     total += t;
-    first += lds_key[o] < key ? t : 0;
+    cost_all += c;
+    first += before ? t : 0;
+    cost_before += before ? c : 0;
   }
   *total_tiles = total;
+  // cut k sits where the cost reaches k/8 of the whole: inside exactly one expert, whose thread places it
+  if (e < E && rows > 0) {
+    const long long mine = moe_tile_cost(rows);
+    const int nt = moe_tile_count(rows);
+    for (int k = 1; k < 8; ++k) {
+      const long long at = (long long)cost_all * k - (long long)cost_before * 8;   // (cost units x 8)
+      if (at >= 0 && at < mine * 8)   // (float: the cut need not be exact, only inside this expert's tiles)
+        cut_q[k] = ((long long)first << kTileQBits) +
+                   (long long)((float)at / (float)(mine * 8) * (float)nt * (float)(1 << kTileQBits));
+    }
+  }
+  __syncthreads();
+  if (e == 0) {
+    const int n = total < max_tiles ? total : max_tiles;
+    cut_q[0] = 0;
+    cut_q[8] = (long long)n << kTileQBits;
+    bool fits = total > 0 && total <= max_tiles;
+    for (int k = 0; k < 8 && fits; ++k) fits = cut_q[k + 1] - cut_q[k] <= moe_xcd_share_cap_q(max_tiles);
+    if (fits) {
+      hdr->n_tiles = n;
+      for (int k = 0; k <= 8; ++k) hdr->xcd_q[k] = cut_q[k];
+    } else {
+      moe_tile_even_shares(hdr, n);   // (a share beyond what the launch provides workgroups for: equal counts always fit)
+    }
+  }
   return first;
 }
 #endif

@@ -83,10 +83,9 @@ __global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __rest
   }
   const int tiles = moe_tile_count(rows);
   int total = 0;
-  const int first = moe_tile_first(e, E, rows, s_rows, s_key, &total);
+  const int first = moe_tile_first(e, E, rows, s_rows, s_key, &total, l.hdr, l.max_tiles);
   for (int t = 0; t < tiles; ++t)
     if (first + t < l.max_tiles) l.tiles[first + t] = TileEntry{e, start, rows, first};   // (cannot overflow for consistent offsets)
-  if (e == 0) l.hdr->n_tiles = total < l.max_tiles ? total : l.max_tiles;
 }
 
 // ---- the kernel ------------------------------------------------------------------------------------------------
@@ -475,13 +474,11 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     int N, void* __restrict__ out, float* __restrict__ out_scale) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   // work items = (row tile, column block) pairs in [expert][column block][row tile] order, dealt to the 8 XCDs in
-  // contiguous ranges (workgroup ids are issued round-robin over XCDs)
+  // contiguous ranges of about equal cost (workgroup ids are issued round-robin over XCDs)
   const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
-  const int n_items = hdr->n_tiles * ncb;
-  const int per_xcd = (n_items + 7) >> 3;
-  const int slot = blockIdx.x >> 3;
-  const int item_id = (blockIdx.x & 7) * per_xcd + slot;
-  if (slot >= per_xcd || item_id >= n_items) return;
+  const int xcd = blockIdx.x & 7;
+  const int item_id = (int)((hdr->xcd_q[xcd] * ncb) >> kTileQBits) + (int)(blockIdx.x >> 3);
+  if (item_id >= (int)((hdr->xcd_q[xcd + 1] * ncb) >> kTileQBits)) return;
   Item item;
   {
     const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
@@ -533,7 +530,8 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
   if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE>, CLS_LDS_BYTES, lds_raised)) return rc;
   const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
   MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
-  const int grid = (int)((max_items + 7) / 8) * 8;   // sized by the worst case; surplus workgroups exit at once
+  // sized by the worst case of the largest XCD share (moe_xcd_share_cap_q); surplus workgroups exit at once
+  const int grid = 8 * (int)((max_items + 7) / 8 + 2);
   hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NT), CLS_LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1,
                      sw1, l.hdr, l.tiles, K, N, out, out_scale);
   return moe_check_hip(hipGetLastError(), "gemm launch");

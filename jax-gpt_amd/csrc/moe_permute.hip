@@ -111,10 +111,9 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
     __syncthreads();   // (tot is read above by nobody else: it doubles as the helper's scratch from here on)
     int all = 0;
     const int nt = e < E ? moe_tile_count(total) : 0;
-    const int first = moe_tile_first(e, E, e < E ? total : 0, tot, tile_key, &all);
+    const int first = moe_tile_first(e, E, e < E ? total : 0, tot, tile_key, &all, tl.hdr, tl.max_tiles);
     for (int t = 0; t < nt; ++t)
       if (first + t < tl.max_tiles) tl.tiles[first + t] = TileEntry{e, excl, total, first};
-    if (e == 0) tl.hdr->n_tiles = all < tl.max_tiles ? all : tl.max_tiles;
   }
 }
 
@@ -219,7 +218,7 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
       if (i < wv) first += wave_tiles[i];
       all += wave_tiles[i];
     }
-    if (threadIdx.x == 0) tl.hdr->n_tiles = all < tl.max_tiles ? all : tl.max_tiles;
+    if (threadIdx.x == 0) moe_tile_even_shares(tl.hdr, all < tl.max_tiles ? all : tl.max_tiles);   // (32-row tiles: all alike)
   }
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
