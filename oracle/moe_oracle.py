@@ -245,7 +245,14 @@ def route_sigmoid_grouped(logits, bias, n_group, topk_group, k, renorm=True, rou
     group's top-2 choice scores; keep the topk_group best groups; top-k experts
     among them by choice score; weights = un-biased scores, renormalised with
     +1e-20, times routed_scale.  Order fixed to value-descending, ties -> lower
-    index (HF leaves it unsorted)."""
+    index (HF leaves it unsorted).
+
+    Masking convention: experts of dropped groups take -inf before the final
+    top-k, as DeepSeek's own inference code does (masked_fill_(..., -inf)); the
+    HF port fills 0.0 instead, which differs only when a kept expert's biased
+    score is negative (a dropped expert's 0.0 would then outrank it).  With
+    -inf a dropped group never contributes an expert as long as the kept
+    groups hold at least k experts."""
     f = np.float32
     logits = np.asarray(logits, dtype=f)
     M, E = logits.shape

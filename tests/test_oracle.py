@@ -453,3 +453,24 @@ def test_continuing_from_given_intermediates_reproduces_the_path():
     cont = O.moe_experts_rows(x, toks, ref["indices"], ref["weights"], fetch, shared=shared, routed_h=rows["routed_h"],
                               shared_h=rows["shared_h"])
     assert np.array_equal(cont, ref["out"][toks])
+
+
+def test_distance_to_the_reference_bf16_activation_dataflow(capsys):
+    """The oracle quantises activations to 1x128 fp8 (x and h); the reference feeds bf16 activations to ragged_dot and
+    accumulates the combine in bf16 (moe.py:83-94).  Parity with the reference itself is unpinned (JAX is not
+    importable here); this reports how far the two arithmetics sit apart on one small layer, through the line-by-line
+    port of the reference's dataflow, and bounds it by what two e4m3 quantisations explain."""
+    from oracle import reference_dataflow as RD
+    x, logits, experts, sh = _tiny_problem(seed=3, M=64, D=512, E=8, k=2, I=256)
+    ours = O.moe_experts(x, logits, experts, top_k=2, shared=sh)["out"]
+    ref = RD.moe_layer_reference(x, logits, experts, 2, shared=sh)
+    err = np.abs(ours - ref)
+    scale = np.abs(ref).max()
+    rel_rows = np.linalg.norm(ours - ref, axis=1) / np.linalg.norm(ref, axis=1)
+    with capsys.disabled():
+        print(f"\n  fp8-activation oracle vs reference bf16-activation dataflow: max|d|/max|ref| = {err.max() / scale:.3e}, "
+              f"row L2 error median {np.median(rel_rows):.3e} / worst {rel_rows.max():.3e}")
+    # an e4m3 value carries 3 mantissa bits (relative step 2^-3 .. 2^-4, rounding error up to 2^-4); errors of
+    # independent elements average down over the K-long dot products, so rows agree to a few percent
+    assert err.max() / scale < 8e-2
+    assert np.median(rel_rows) < 6e-2
