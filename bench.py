@@ -164,10 +164,13 @@ def run_workload(jg, torch, name, cfg, layer, steps, warmup):
     # stream it is launched on (torch's current stream is the stream handed to the C ABI)
     sg = jg.permute(dbg["indices"], E)
     xq, sx = jg.quant_act(x)
+    # as moe_forward launches it: large batches read their activation scales block-major, in sorted row order
+    blocked = R > 2048
+    sxk = jg.gather_scales(sx, sg["sorted_token_ids"]) if blocked else sx
 
     def gateup():
-        jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], sg["group_offsets"],
-                              row_ids=sg["sorted_token_ids"])
+        jg.gemm_gateup_swiglu(xq, sxk, experts["gate_proj"], experts["up_proj"], sg["group_offsets"],
+                              row_ids=sg["sorted_token_ids"], block_major=blocked)
 
     k_ms, _ = timed(torch, gateup, steps, max(2, warmup // 2))
     k_flops = 4.0 * R * D * I
@@ -200,17 +203,19 @@ def run_ep_shard(jg, torch, steps, warmup, seed=5):
     xq, sx = jg.quant_act(torch.randn((R, D), dtype=torch.float32, device="cuda", generator=gen).to(torch.bfloat16))
     log(f"ep_shard_skewed: rows per expert, ascending: {sorted(int(v) for v in group_sizes)}")
 
-    def step():
-        hq, sh = jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], off)
-        y = jg.gemm_down(hq, sh, experts["down_proj"], off)
+    def step():   # (the rows arrive with row-major scales, as a dispatch all-to-all delivers them: the gather is part of the step)
+        sxb = jg.gather_scales(sx)
+        hq, sh = jg.gemm_gateup_swiglu(xq, sxb, experts["gate_proj"], experts["up_proj"], off, block_major=True)
+        y = jg.gemm_down(hq, sh, experts["down_proj"], off, block_major=True)
         return jg.combine(y, weights, inv_perm)
 
     out = step()
     torch.cuda.synchronize()
     assert torch.isfinite(out.float()).all(), "non-finite output"
     ms, _ = timed(torch, step, steps, warmup)
-    k_ms, _ = timed(torch, lambda: jg.gemm_gateup_swiglu(xq, sx, experts["gate_proj"], experts["up_proj"], off), steps,
-                    max(2, warmup // 2))
+    sxb = jg.gather_scales(sx)
+    k_ms, _ = timed(torch, lambda: jg.gemm_gateup_swiglu(xq, sxb, experts["gate_proj"], experts["up_proj"], off,
+                                                         block_major=True), steps, max(2, warmup // 2))
     flops = 6.0 * R * D * I
     k_flops = 4.0 * R * D * I
     touched = int((group_sizes > 0).sum())

@@ -108,10 +108,32 @@ MOE_API int moe_gemm_gateup_swiglu_fp8_static(const uint8_t* xq, const float* sx
                                       const int32_t* group_offsets, int E, int R, int D, int I,
                                       uint8_t* hq, float* sh, moe_stream_t stream);
 
+/* Scale layouts of the grouped GEMMs' activation operands (no counterpart in the reference, which has no
+ * activation scales).  ROW_MAJOR is what the quantisers write: (rows, K/128), indexed through row_ids like the
+ * codes.  BLOCK_MAJOR is (K/128, R) in row-list order (entry [kb][p] belongs to list position p; row_ids is not
+ * applied to it): a K step of a 256-row tile then reads its row scales from 8 cache lines instead of 256, which
+ * is worth 2-3 % of the GEMM time at prefill sizes.  moe_gather_scales makes the block-major array from the
+ * row-major one; moe_forward does this by itself for batches of more than 2048 routed rows. */
+#define MOE_SCALES_ROW_MAJOR 0
+#define MOE_SCALES_BLOCK_MAJOR 1
+MOE_API int moe_gather_scales(const float* sx, const int32_t* row_ids, int R, int KB, float* out,
+                              moe_stream_t stream);
+/* moe_gemm_gateup_swiglu_fp8 with the layout of sx (read) and of sh (written) chosen by the caller. */
+MOE_API int moe_gemm_gateup_swiglu_fp8_layout(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+                                      const uint8_t* w_gate, const float* sw_gate,
+                                      const uint8_t* w_up, const float* sw_up,
+                                      const int32_t* group_offsets, int E, int R, int D, int I,
+                                      uint8_t* hq, float* sh, void* ws, size_t ws_bytes,
+                                      int sx_layout, int sh_layout, moe_stream_t stream);
+
 /* moe.py:87 (the third ragged_dot): y = h . Wdown[e]^T, bf16 out (R, D). */
 MOE_API int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down,
                       const float* sw_down, const int32_t* group_offsets, int E, int R, int I,
                       int D, void* y_bf16, void* ws, size_t ws_bytes, moe_stream_t stream);
+/* The same with sh in the given layout (MOE_SCALES_*). */
+MOE_API int moe_gemm_down_fp8_layout(const uint8_t* hq, const float* sh, const uint8_t* w_down,
+                      const float* sw_down, const int32_t* group_offsets, int E, int R, int I,
+                      int D, void* y_bf16, void* ws, size_t ws_bytes, int sh_layout, moe_stream_t stream);
 
 /* moe.py:90-94 (_scatter_back) as a deterministic gather: out[t] = sum_s w[t,s] *
  * y[inv_perm[t*k+s]] (+ shared_gate[t] * shared[t]) in f32, one bf16 rounding.  shared may be

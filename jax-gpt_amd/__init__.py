@@ -9,6 +9,7 @@ the built library and a GPU every compute call raises.
 from ._lib import lib, MoeError  # noqa: F401
 from .moe import (  # noqa: F401
     convert,
+    gather_scales,
     block_fp8_from_per_row,
     combine,
     expert_forward_single,

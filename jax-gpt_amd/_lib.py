@@ -56,6 +56,9 @@ SIGNATURES = {
     "moe_gemm_gateup_swiglu_fp8": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _Z, _P]),
     "moe_gemm_gateup_swiglu_fp8_static": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]),
     "moe_gemm_down_fp8": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _Z, _P]),
+    "moe_gemm_gateup_swiglu_fp8_layout": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P, _Z, _I, _I, _P]),
+    "moe_gemm_down_fp8_layout": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P, _P, _Z, _I, _P]),
+    "moe_gather_scales": (_I, [_P, _P, _I, _I, _P, _P]),
     "moe_combine": (_I, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P, _P]),
     "moe_rmsnorm_quant": (_I, [_P, _P, _F, _I, _I, _P, _P, _P, _P]),
     "moe_router_workspace_bytes": (_Z, [_I, _I, _I]),

@@ -24,7 +24,7 @@ int moe_check_hip(hipError_t e, const char* what) {
   return moe_set_error(MOE_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
-extern "C" int moe_abi_version(void) { return 5; }
+extern "C" int moe_abi_version(void) { return 6; }
 extern "C" const char* moe_last_error(void) { return g_err; }
 
 namespace {
@@ -65,7 +65,7 @@ struct Carver {
 
 struct ForwardBuffers {
   int32_t *idx, *group_sizes, *group_offsets, *sorted_token_ids, *inv_perm, *dense_off;
-  float *w, *sx, *sh, *shs, *shared_gate;
+  float *w, *sx, *sh, *shs, *shared_gate, *sx_listed, *sx_blocked;
   uint8_t *xq, *hq, *hsq;
   void *y, *ys, *permute_ws, *gemm_ws, *gemm_ws_shared, *router_ws, *normed;
   size_t permute_ws_bytes, gemm_ws_bytes, gemm_ws_shared_bytes, router_ws_bytes, total;
@@ -91,6 +91,10 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool r
   b.gemm_ws_shared = SI ? c.take(b.gemm_ws_shared_bytes) : nullptr;
   b.xq = (uint8_t*)c.take((size_t)M * D);
   b.sx = (float*)c.take((size_t)M * (D / 128) * 4);
+  // block-major copies of the activation scales for large batches (GemmScales): routed rows in sorted order,
+  // and the tokens in their own order for the shared expert
+  b.sx_listed = (float*)c.take(R * (D / 128) * 4);
+  b.sx_blocked = SI ? (float*)c.take((size_t)M * (D / 128) * 4) : nullptr;
   b.hq = (uint8_t*)c.take(R * I);
   b.sh = (float*)c.take(R * (I / 128) * 4);
   b.y = c.take(R * D * 2);
@@ -161,6 +165,9 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   void* y = a->out_y ? a->out_y : b.y;
   void* ys = a->out_ys ? a->out_ys : b.ys;
   const int R = a->M * a->k;
+  // large batches read their activation scales from block-major arrays (GemmScales); a decode-sized batch touches
+  // few scale lines either way and is spared the extra launch
+  const bool blocked_scales = R > 2048;
   hipStream_t main_s = (hipStream_t)stream;
   MOE_REQUIRE(a->routing == MOE_ROUTING_SOFTMAX || a->routing == MOE_ROUTING_SIGMOID_GROUPED, MOE_ERR_BAD_SHAPE,
               "forward: unknown routing %d", a->routing);
@@ -191,13 +198,22 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     rc_shared = quantise(a, b, (moe_stream_t)side);
     if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
+    GemmScales sc = moe_row_major_scales(a->D, a->SI);
+    const float* sx_shared = b.sx;
+    if (blocked_scales) {
+      if (!rc_shared) rc_shared = moe_gather_scales(b.sx, nullptr, a->M, a->D / 128, b.sx_blocked, (moe_stream_t)side);
+      sx_shared = b.sx_blocked;
+      sc.in_row = 1, sc.in_kb = a->M, sc.in_listed = true;
+      if (!a->out_shs) sc.out_row = 1, sc.out_cb = a->M;   // (a debug copy of the h scales keeps the documented layout)
+    }
     if (!rc_shared)
-      rc_shared = moe_gemm_gateup_impl(b.xq, b.sx, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up, b.dense_off, 1,
-                                       a->M, a->D, a->SI, hsq, shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, false,
+      rc_shared = moe_gemm_gateup_impl(b.xq, sx_shared, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up, b.dense_off,
+                                       1, a->M, a->D, a->SI, hsq, shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, false, sc,
                                        (moe_stream_t)side);
     if (!rc_shared)   // same rows, same tile height: the list the gate/up launch built serves the down launch too
       rc_shared = moe_gemm_down_impl(hsq, shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, ys,
-                                     b.gemm_ws_shared, b.gemm_ws_shared_bytes, true, (moe_stream_t)side);
+                                     b.gemm_ws_shared, b.gemm_ws_shared_bytes, true,
+                                     GemmScales{sc.out_row, sc.out_cb, true, 0, 0}, (moe_stream_t)side);
   } else {
     if ((rc = quantise(a, b, stream))) return rc;
   }
@@ -256,11 +272,19 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     if (rc_shared) return join(rc_shared);
     if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
   }
-  if ((rc = moe_gemm_gateup_impl(b.xq, b.sx, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets, a->E, R,
-                                 a->D, a->I, hq, sh, b.gemm_ws, b.gemm_ws_bytes, true, stream)))
+  GemmScales sc = moe_row_major_scales(a->D, a->I);
+  const float* sx_routed = b.sx;
+  if (blocked_scales) {
+    if ((rc = moe_gather_scales(b.sx, stid, R, a->D / 128, b.sx_listed, stream))) return join(rc);
+    sx_routed = b.sx_listed;
+    sc.in_row = 1, sc.in_kb = R, sc.in_listed = true;
+    if (!a->out_sh) sc.out_row = 1, sc.out_cb = R;
+  }
+  if ((rc = moe_gemm_gateup_impl(b.xq, sx_routed, stid, a->w_gate, a->sw_gate, a->w_up, a->sw_up, b.group_offsets, a->E,
+                                 R, a->D, a->I, hq, sh, b.gemm_ws, b.gemm_ws_bytes, true, sc, stream)))
     return join(rc);
   if ((rc = moe_gemm_down_impl(hq, sh, a->w_down, a->sw_down, b.group_offsets, a->E, R, a->I, a->D, y,
-                               b.gemm_ws, b.gemm_ws_bytes, true, stream)))
+                               b.gemm_ws, b.gemm_ws_bytes, true, GemmScales{sc.out_row, sc.out_cb, true, 0, 0}, stream)))
     return join(rc);
   if ((rc = join(MOE_OK))) return rc;
   return moe_combine(y, w, inv, a->SI ? ys : nullptr, shared_gate, a->add_residual ? a->x : nullptr, a->M, a->k,

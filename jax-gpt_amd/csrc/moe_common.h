@@ -183,13 +183,24 @@ int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list);
 int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_sizes, int32_t* group_offsets,
                      int32_t* sorted_token_ids, int32_t* sort_order, int32_t* inv_perm, void* ws, size_t ws_bytes,
                      TileList tiles, moe_stream_t stream);
+// Where the grouped GEMMs find an activation scale and put an h scale, in floats: scale of (row, 128-wide K block kb)
+// = s[row * in_row + kb * in_kb].  The public entry points use the row-major arrays of the quantisers ({K/128, 1});
+// moe_forward hands large batches block-major arrays in row-list order ({1, R}, in_listed = true: indexed by the
+// position in the row list, not through row_ids), because a K step then reads its 256 row scales from 8 lines
+// instead of 256 (a 4-byte read costs the vector L1 a whole line request: -2 to -3 % GEMM time).
+struct GemmScales {
+  int in_row, in_kb;
+  bool in_listed;
+  int out_row, out_cb;   // gate/up only: scale of (row, column block cb) of h = sh[row * out_row + cb * out_cb]
+};
+inline GemmScales moe_row_major_scales(int K, int I) { return GemmScales{K / 128, 1, false, I / 128, 1}; }
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
                          const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
                          int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,
-                         moe_stream_t stream);
+                         GemmScales sc, moe_stream_t stream);
 int moe_gemm_down_impl(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
                        const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
-                       size_t ws_bytes, bool list_built, moe_stream_t stream);
+                       size_t ws_bytes, bool list_built, GemmScales sc, moe_stream_t stream);
 
 #define MOE_REQUIRE(cond, code, ...) \
   do {                               \

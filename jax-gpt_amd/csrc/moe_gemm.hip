@@ -149,7 +149,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
                                           const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
                                           const uint8_t* __restrict__ w0, const float* __restrict__ sw0,
                                           const uint8_t* __restrict__ w1, const float* __restrict__ sw1, int K, int N,
-                                          void* __restrict__ out, float* __restrict__ out_scale) {
+                                          void* __restrict__ out, float* __restrict__ out_scale, const GemmScales sc) {
   using C = Cls<XF>;
   constexpr int BM = C::BM, HALF = C::HALF;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -189,8 +189,8 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
     const int q = p % HALF;
     const int r = 16 * (2 * (q % XF) + p / HALF) + q / XF;
     int g = item.row_start + min(r, item.row_count - 1);
-    if (row_ids) g = row_ids[g];
-    soff = (unsigned)g * (unsigned)KB * 4u;
+    if (row_ids && !sc.in_listed) g = row_ids[g];
+    soff = (unsigned)g * (unsigned)sc.in_row * 4u;
   }
   const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);
   auto issue_op = [&](int kb, int i) {
@@ -200,7 +200,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
       int grp = (i - 4) * NWAVES + wave;
       if (grp >= C::X_GROUPS) grp -= 4;
       dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + grp * 1024u);
-    } else dma4((const uint8_t*)(sx + kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4u);
+    } else dma4((const uint8_t*)(sx + (size_t)kb * sc.in_kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4u);
   };
 #pragma unroll
   for (int s = 0; s < C::PRE; ++s)
@@ -423,7 +423,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
         *(unsigned*)(tile + swz(xr, col >> 4) + (col & 15)) = q;
       }
       if (wi == 0 && fq == 0 && xr < item.row_count)
-        out_scale[(size_t)(item.row_start + xr) * (I / 128) + item.col_block] = scale_inv;
+        out_scale[(size_t)(item.row_start + xr) * sc.out_row + (size_t)item.col_block * sc.out_cb] = scale_inv;
     }
     __syncthreads();
     const int ld_chunk = tid & 7, ld_row = tid >> 3;   // 64 rows per pass
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0, const uint8_t* __restrict__ w1,
     const float* __restrict__ sw1, const TileHeader* __restrict__ hdr, const TileEntry* __restrict__ tiles, int K,
-    int N, void* __restrict__ out, float* __restrict__ out_scale) {
+    int N, void* __restrict__ out, float* __restrict__ out_scale, const GemmScales sc) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   // work items = (row tile, column block) pairs in [expert][column block][row tile] order, dealt to the 8 XCDs in
   // contiguous ranges of about equal cost (workgroup ids are issued round-robin over XCDs)
@@ -519,7 +519,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     item.row_count = tn;
   }
   const int rows = __builtin_amdgcn_readfirstlane(item.row_count);
-#define MOE_ITEM(XF) item_body<MODE, XF>(item, lds, xq, sx, row_ids, w0, sw0, w1, sw1, K, N, out, out_scale)
+#define MOE_ITEM(XF) item_body<MODE, XF>(item, lds, xq, sx, row_ids, w0, sw0, w1, sw1, K, N, out, out_scale, sc)
   switch ((rows + 31) >> 5) {
     case 8: MOE_ITEM(8); break;
     case 7: MOE_ITEM(7); break;
@@ -543,7 +543,7 @@ TileList tile_list(void* ws, int R, int E) {
 template <int MODE>
 int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w0, const float* sw0,
            const uint8_t* w1, const float* sw1, const int32_t* group_offsets, int E, int R, int K, int N,
-           void* out, float* out_scale, void* ws, size_t ws_bytes, bool list_built, hipStream_t s) {
+           void* out, float* out_scale, void* ws, size_t ws_bytes, bool list_built, GemmScales sc, hipStream_t s) {
   const size_t need = moe_gemm_workspace_bytes(R, E, N);
   MOE_REQUIRE(ws_bytes >= need, MOE_ERR_WORKSPACE_TOO_SMALL, "gemm: workspace %zu < %zu", ws_bytes, need);
   MOE_REQUIRE(K <= MAX_KB * BK, MOE_ERR_BAD_SHAPE, "gemm: contraction length %d exceeds %d", K, MAX_KB * BK);
@@ -559,7 +559,7 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
   // sized by the worst case of the largest XCD share (moe_xcd_share_cap_q); surplus workgroups exit at once
   const int grid = 8 * (int)((max_items + 7) / 8 + 2);
   hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NT), CLS_LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1,
-                     sw1, l.hdr, l.tiles, K, N, out, out_scale);
+                     sw1, l.hdr, l.tiles, K, N, out, out_scale, sc);
   return moe_check_hip(hipGetLastError(), "gemm launch");
 }
 
@@ -573,15 +573,17 @@ extern "C" size_t moe_gemm_workspace_bytes(int R, int E, int N_out) {
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
                          const float* sw_gate, const uint8_t* w_up, const float* sw_up, const int32_t* group_offsets,
                          int E, int R, int D, int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, bool list_built,
-                         moe_stream_t stream) {
+                         GemmScales sc, moe_stream_t stream) {
   MOE_REQUIRE((R == 0 || (xq && sx && hq && sh)) && w_gate && sw_gate && w_up && sw_up && group_offsets && ws, MOE_ERR_NULL,
               "gemm_gateup: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0 && D > 0 && I > 0 && D % 128 == 0 && I % 128 == 0, MOE_ERR_BAD_SHAPE,
               "gemm_gateup: need D %% 128 == 0 and I %% 128 == 0 and 1 <= E <= 1024, got E=%d R=%d D=%d I=%d", E, R, D, I);
   MOE_REQUIRE(MOE_ALIGNED16(xq) && MOE_ALIGNED16(w_gate) && MOE_ALIGNED16(w_up) && MOE_ALIGNED16(hq) && MOE_ALIGNED16(ws),
               MOE_ERR_BAD_ALIGN, "gemm_gateup: pointers must be 16-byte aligned");
+  MOE_REQUIRE((long long)R * sc.in_row * 4 <= (1ll << 32) && (long long)R * sc.out_row + (long long)(I / 128) * sc.out_cb <= (1ll << 40),
+              MOE_ERR_BAD_SHAPE, "gemm_gateup: scale array out of the addressable range");
   return launch<MODE_GATEUP>(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
-                             ws_bytes, list_built, (hipStream_t)stream);
+                             ws_bytes, list_built, sc, (hipStream_t)stream);
 }
 
 extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, const int32_t* row_ids,
@@ -590,7 +592,29 @@ extern "C" int moe_gemm_gateup_swiglu_fp8(const uint8_t* xq, const float* sx, co
                                           int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes,
                                           moe_stream_t stream) {
   return moe_gemm_gateup_impl(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
-                              ws_bytes, false, stream);
+                              ws_bytes, false, moe_row_major_scales(D, I), stream);
+}
+
+namespace {
+int check_layout(int layout, const char* what) {
+  MOE_REQUIRE(layout == MOE_SCALES_ROW_MAJOR || layout == MOE_SCALES_BLOCK_MAJOR, MOE_ERR_BAD_SHAPE,
+              "%s: unknown scale layout %d", what, layout);
+  return MOE_OK;
+}
+}  // namespace
+
+extern "C" int moe_gemm_gateup_swiglu_fp8_layout(const uint8_t* xq, const float* sx, const int32_t* row_ids,
+                                                 const uint8_t* w_gate, const float* sw_gate, const uint8_t* w_up,
+                                                 const float* sw_up, const int32_t* group_offsets, int E, int R, int D,
+                                                 int I, uint8_t* hq, float* sh, void* ws, size_t ws_bytes, int sx_layout,
+                                                 int sh_layout, moe_stream_t stream) {
+  if (int rc = check_layout(sx_layout, "gemm_gateup: sx")) return rc;
+  if (int rc = check_layout(sh_layout, "gemm_gateup: sh")) return rc;
+  GemmScales sc = moe_row_major_scales(D, I);
+  if (sx_layout == MOE_SCALES_BLOCK_MAJOR) sc.in_row = 1, sc.in_kb = R, sc.in_listed = true;
+  if (sh_layout == MOE_SCALES_BLOCK_MAJOR) sc.out_row = 1, sc.out_cb = R;
+  return moe_gemm_gateup_impl(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
+                              ws_bytes, false, sc, stream);
 }
 
 namespace {
@@ -627,26 +651,37 @@ extern "C" int moe_gemm_gateup_swiglu_fp8_static(const uint8_t* xq, const float*
   // the tile list (header and every entry the GEMM reads) is rewritten by this call's first kernel: nothing of
   // an earlier call's contents is read
   return moe_gemm_gateup_impl(xq, sx, row_ids, w_gate, sw_gate, w_up, sw_up, group_offsets, E, R, D, I, hq, sh, ws,
-                              MOE_STATIC_SCRATCH_BYTES, false, stream);
+                              MOE_STATIC_SCRATCH_BYTES, false, moe_row_major_scales(D, I), stream);
 }
 
 int moe_gemm_down_impl(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
                        const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
-                       size_t ws_bytes, bool list_built, moe_stream_t stream) {
+                       size_t ws_bytes, bool list_built, GemmScales sc, moe_stream_t stream) {
   MOE_REQUIRE((R == 0 || (hq && sh && y_bf16)) && w_down && sw_down && group_offsets && ws, MOE_ERR_NULL,
               "gemm_down: null pointer");
   MOE_REQUIRE(E >= 1 && E <= 1024 && R >= 0 && D > 0 && I > 0 && D % 128 == 0 && I % 128 == 0, MOE_ERR_BAD_SHAPE,
               "gemm_down: need D %% 128 == 0 and I %% 128 == 0 and 1 <= E <= 1024, got E=%d R=%d I=%d D=%d", E, R, I, D);
   MOE_REQUIRE(MOE_ALIGNED16(hq) && MOE_ALIGNED16(w_down) && MOE_ALIGNED16(y_bf16) && MOE_ALIGNED16(ws), MOE_ERR_BAD_ALIGN,
               "gemm_down: pointers must be 16-byte aligned");
+  MOE_REQUIRE((long long)R * sc.in_row * 4 <= (1ll << 32), MOE_ERR_BAD_SHAPE, "gemm_down: scale array out of the addressable range");
   return launch<MODE_DOWN>(hq, sh, nullptr, w_down, sw_down, nullptr, nullptr, group_offsets, E, R, I, D, y_bf16,
-                           nullptr, ws, ws_bytes, list_built, (hipStream_t)stream);
+                           nullptr, ws, ws_bytes, list_built, sc, (hipStream_t)stream);
 }
 
 extern "C" int moe_gemm_down_fp8(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
                                  const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16, void* ws,
                                  size_t ws_bytes, moe_stream_t stream) {
-  return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, stream);
+  return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false,
+                            moe_row_major_scales(I, D), stream);
+}
+
+extern "C" int moe_gemm_down_fp8_layout(const uint8_t* hq, const float* sh, const uint8_t* w_down, const float* sw_down,
+                                        const int32_t* group_offsets, int E, int R, int I, int D, void* y_bf16,
+                                        void* ws, size_t ws_bytes, int sh_layout, moe_stream_t stream) {
+  if (int rc = check_layout(sh_layout, "gemm_down: sh")) return rc;
+  GemmScales sc = moe_row_major_scales(I, D);
+  if (sh_layout == MOE_SCALES_BLOCK_MAJOR) sc.in_row = 1, sc.in_kb = R, sc.in_listed = true;
+  return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, sc, stream);
 }
 
 // The tile list that the GEMM launches of (R rows, E experts) read from ws when they are told list_built = true.

@@ -193,3 +193,35 @@ extern "C" int moe_convert(const void* src, int src_is_f32, void* dst, int dst_i
                      dst, dst_is_f32, n);
   return moe_check_hip(hipGetLastError(), "convert launch");
 }
+
+namespace {
+// Activation scales, row-major (rows, KB) -> block-major (KB, n) in row-list order: out[kb][p] = sx[ids ? ids[p] : p][kb].
+// One thread per list position: it reads its row's KB scales (one or two lines) and writes one float into each of the
+// KB output rows, where neighbouring threads write neighbouring floats.
+__global__ __launch_bounds__(256) void gather_scales_kernel(const float* __restrict__ sx, const int32_t* __restrict__ ids,
+                                                           int n, int KB, float* __restrict__ out) {
+  const int p = blockIdx.x * 256 + threadIdx.x;
+  if (p >= n) return;
+  const float* src = sx + (size_t)(ids ? ids[p] : p) * KB;
+  int kb = 0;
+  if ((KB & 3) == 0) {
+    for (; kb < KB; kb += 4) {
+      const float4 v = *(const float4*)(src + kb);
+      out[(size_t)kb * n + p] = v.x;
+      out[(size_t)(kb + 1) * n + p] = v.y;
+      out[(size_t)(kb + 2) * n + p] = v.z;
+      out[(size_t)(kb + 3) * n + p] = v.w;
+    }
+  }
+  for (; kb < KB; ++kb) out[(size_t)kb * n + p] = src[kb];
+}
+}  // namespace
+
+extern "C" int moe_gather_scales(const float* sx, const int32_t* row_ids, int n, int KB, float* out, moe_stream_t stream) {
+  MOE_REQUIRE(n >= 0 && KB >= 1, MOE_ERR_BAD_SHAPE, "gather_scales: bad sizes n=%d KB=%d", n, KB);
+  MOE_REQUIRE(n == 0 || (sx && out), MOE_ERR_NULL, "gather_scales: null pointer");
+  if (n == 0) return MOE_OK;
+  hipLaunchKernelGGL(gather_scales_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, sx, row_ids,
+                     n, KB, out);
+  return moe_check_hip(hipGetLastError(), "gather_scales launch");
+}

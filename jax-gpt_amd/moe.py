@@ -259,9 +259,28 @@ def _gemm_ws(R, E, n_out, like):
     return _empty((nbytes,), torch.uint8, like), nbytes
 
 
-def gemm_gateup_swiglu(xq, sx, gate, up, group_offsets, row_ids=None, n_rows=None):
+SCALES_ROW_MAJOR, SCALES_BLOCK_MAJOR = 0, 1
+
+
+def gather_scales(sx, row_ids=None, n_rows=None):
+    """Row-major activation scales (rows, KB) -> block-major (KB, R) in row-list order:
+    out[kb, p] = sx[row_ids[p], kb] (row_ids None: p).  The layout the grouped GEMMs read fastest."""
+    sx = _dev(sx, torch.float32, "sx")
+    if row_ids is not None:
+        row_ids = _dev(row_ids, torch.int32, "row_ids")
+        R = row_ids.numel() if n_rows is None else n_rows
+    else:
+        R = sx.shape[0] if n_rows is None else n_rows
+    KB = sx.shape[1]
+    out = _empty((KB, R), torch.float32, sx)
+    check(lib().moe_gather_scales(_ptr(sx), _ptr(row_ids), R, KB, _ptr(out), _stream()))
+    return out
+
+
+def gemm_gateup_swiglu(xq, sx, gate, up, group_offsets, row_ids=None, n_rows=None, block_major=False):
     """h = silu(x.Wg^T) * (x.Wu^T) per expert row range, quantised 1x128 -> (hq, sh).
-    row_ids maps sorted position -> row of xq (None: rows are already in expert order)."""
+    row_ids maps sorted position -> row of xq (None: rows are already in expert order).
+    block_major: sx is a gather_scales() array (KB, R) and sh comes back as (I/128, R)."""
     xq = _codes(xq, "xq")
     sx = _dev(sx, torch.float32, "sx")
     wg, sg = _expert_weight(gate, "gate_proj")
@@ -278,15 +297,23 @@ def gemm_gateup_swiglu(xq, sx, gate, up, group_offsets, row_ids=None, n_rows=Non
     else:
         R = xq.shape[0] if n_rows is None else n_rows
     hq = _empty((R, I), torch.uint8, xq)
-    sh = _empty((R, I // 128), torch.float32, xq)
     ws, nbytes = _gemm_ws(R, E, I, xq)
+    if block_major:
+        if tuple(sx.shape) != (D // 128, R):
+            raise ValueError(f"block-major sx must be {(D // 128, R)}, got {tuple(sx.shape)}")
+        sh = _empty((I // 128, R), torch.float32, xq)
+        check(lib().moe_gemm_gateup_swiglu_fp8_layout(_ptr(xq), _ptr(sx), _ptr(row_ids), _ptr(wg), _ptr(sg), _ptr(wu),
+                                                      _ptr(su), _ptr(go), E, R, D, I, _ptr(hq), _ptr(sh), _ptr(ws), nbytes,
+                                                      SCALES_BLOCK_MAJOR, SCALES_BLOCK_MAJOR, _stream()))
+        return hq.view(torch.float8_e4m3fn), sh
+    sh = _empty((R, I // 128), torch.float32, xq)
     check(lib().moe_gemm_gateup_swiglu_fp8(_ptr(xq), _ptr(sx), _ptr(row_ids), _ptr(wg), _ptr(sg), _ptr(wu), _ptr(su),
                                            _ptr(go), E, R, D, I, _ptr(hq), _ptr(sh), _ptr(ws), nbytes, _stream()))
     return hq.view(torch.float8_e4m3fn), sh
 
 
-def gemm_down(hq, sh, down, group_offsets):
-    """y = h . Wdown[e]^T per expert row range, bf16 (R, D)."""
+def gemm_down(hq, sh, down, group_offsets, block_major=False):
+    """y = h . Wdown[e]^T per expert row range, bf16 (R, D).  block_major: sh is (I/128, R)."""
     hq = _codes(hq, "hq")
     sh = _dev(sh, torch.float32, "sh")
     wd, sd = _expert_weight(down, "down_proj")
@@ -297,6 +324,12 @@ def gemm_down(hq, sh, down, group_offsets):
     go = _dev(group_offsets, torch.int32, "group_offsets")
     y = _empty((R, D), torch.bfloat16, hq)
     ws, nbytes = _gemm_ws(R, E, D, hq)
+    if block_major:
+        if tuple(sh.shape) != (I // 128, R):
+            raise ValueError(f"block-major sh must be {(I // 128, R)}, got {tuple(sh.shape)}")
+        check(lib().moe_gemm_down_fp8_layout(_ptr(hq), _ptr(sh), _ptr(wd), _ptr(sd), _ptr(go), E, R, I, D, _ptr(y),
+                                             _ptr(ws), nbytes, SCALES_BLOCK_MAJOR, _stream()))
+        return y
     check(lib().moe_gemm_down_fp8(_ptr(hq), _ptr(sh), _ptr(wd), _ptr(sd), _ptr(go), E, R, I, D, _ptr(y), _ptr(ws),
                                   nbytes, _stream()))
     return y

@@ -32,7 +32,7 @@ def test_header_and_library_agree(dll):
     for name in declared:
         assert hasattr(dll, name), f"{name} is declared in moe_hip.h but not exported"
     assert sorted(_lib.SIGNATURES) == declared
-    assert dll.moe_abi_version() == 5
+    assert dll.moe_abi_version() == 6
 
 
 def test_library_exports_exactly_the_header(dll):

@@ -141,6 +141,47 @@ def _ragged_case(seed, E, D, I, sizes):
     return off, xq, sx, dict(gate=mk(I, D), up=mk(I, D), down=mk(D, I))
 
 
+@pytest.mark.parametrize("E,D,I,sizes,gather", [
+    (4, 512, 256, [130, 0, 5, 128], False),
+    (6, 2048, 768, [300, 0, 0, 129, 7, 64], True),
+    (3, 384, 384, [257, 0, 1], True),
+])
+def test_block_major_scales_give_the_same_bits(jg, E, D, I, sizes, gather):
+    """The grouped GEMMs read activation scales row-major (rows, K/128) or block-major (K/128, R) in row-list order
+    (moe_gather_scales; what moe_forward uses for large batches): same codes, same scales, same y, bit for bit.
+    gather: the rows are reached through row_ids (a permutation of a larger array), else they are in expert order."""
+    import torch
+    _say("block_major_scales", E, D, I, sizes, gather)
+    off, xq, sx, ex = _ragged_case(900 + D + I, E, D, I, sizes)
+    R = int(off[-1])
+    dex = H.experts_to_cuda(ex)
+    dxq, dsx, doff = H.to_cuda(xq), H.to_cuda(sx), H.to_cuda(off)
+    ids = None
+    if gather:                                      # hide the rows in a larger array, in shuffled order
+        rng = np.random.default_rng(5)
+        perm = rng.permutation(R + 37).astype(np.int32)[:R]
+        big_q = torch.zeros((R + 37, D), dtype=torch.uint8, device="cuda")
+        big_s = torch.ones((R + 37, D // 128), dtype=torch.float32, device="cuda")
+        ids = torch.from_numpy(perm).cuda()
+        big_q[ids.long()] = dxq.view(torch.uint8)
+        big_s[ids.long()] = dsx
+        dxq, dsx = big_q, big_s
+    hq0, sh0 = jg.gemm_gateup_swiglu(dxq, dsx, dex["gate_proj"], dex["up_proj"], doff, row_ids=ids)
+    sxb = jg.gather_scales(dsx, ids)
+    assert tuple(sxb.shape) == (D // 128, R)
+    want = dsx[ids.long()] if gather else dsx
+    assert torch.equal(sxb, want.t().contiguous())
+    hq1, sh1 = jg.gemm_gateup_swiglu(dxq, sxb, dex["gate_proj"], dex["up_proj"], doff, row_ids=ids, block_major=True)
+    assert tuple(sh1.shape) == (I // 128, R)
+    assert torch.equal(hq0.view(torch.uint8), hq1.view(torch.uint8))
+    assert torch.equal(sh0, sh1.t().contiguous())
+    y0 = jg.gemm_down(hq0, sh0, dex["down_proj"], doff)
+    y1 = jg.gemm_down(hq1, sh1, dex["down_proj"], doff, block_major=True)
+    assert torch.equal(y0.view(torch.int16), y1.view(torch.int16))
+    with pytest.raises(ValueError):
+        jg.gemm_down(hq1, sh0, dex["down_proj"], doff, block_major=True)
+
+
 @pytest.mark.parametrize("E,D,I,sizes", [
     (1, 128, 128, [16]),
     (1, 256, 128, [1]),
