@@ -191,6 +191,7 @@ def test_block_major_scales_give_the_same_bits(jg, E, D, I, sizes, gather):
     (6, 2048, 768, [300, 0, 0, 129, 7, 64]),
     (8, 256, 256, [70, 0, 1, 33, 0, 16, 0, 0]),   # a few rows per expert: the 32- and 64-row tile classes, empty experts between
     (2, 256, 256, [300, 150]),                    # two row tiles for one expert (near-equal cut), one 160-row tile for the other
+    (2, 256, 256, [4200, 100]),                   # 17 row tiles: the column blocks are walked once per group of 8-9 row tiles
 ])
 def test_grouped_gemms_vs_oracle(jg, E, D, I, sizes):
     _say("grouped_gemm", E, D, I, sizes)
