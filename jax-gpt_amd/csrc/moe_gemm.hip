@@ -26,17 +26,16 @@
 // 16-row activation fragments 2j + xj (alternating between the two wave sets, so
 // a short tile still splits evenly).
 //
-// What bounds a work item.  One CU draws at most about 22 GB/s from HBM and about
-// 85 GB/s from its XCD's L2 through its vector L1, however many copies it keeps in
-// flight (measured with a streaming workgroup of this kernel's copy pattern; all
-// 256 CUs together reach the HBM rate).  A K step of a full tile moves 64 KB into
-// LDS and holds 2048 matrix-core cycles per SIMD: the activation tile is shared by
-// the item's 16 column blocks and comes from L2, the weight tile comes from L2 when
-// a neighbouring row tile of the same expert has just fetched it and from HBM
-// otherwise (always, for an expert of one row tile).  An expert of few rows is
-// therefore a weight stream at the per-CU HBM rate whatever the kernel does with
-// its rows; the kernel's part is to keep that stream and the large experts'
-// matrix work going side by side on different CUs, and to waste neither.
+// What bounds a work item.  A K step of a full tile moves 64 KB into LDS (72 copy instructions per CU) and holds
+// 2048 matrix-core cycles per SIMD.  The L2 can fill one CU's LDS at about 125 GB/s with this copy pattern (all CUs
+// at once); a CU streaming alone from HBM gets about 22 GB/s whatever its queue depth, and all 256 together reach
+// the memory's rate.  The activation tile is shared by the item's 16 column blocks and comes from L2, the weight
+// tile comes from L2 when a neighbouring row tile of the same expert has just fetched it and from HBM or the
+// memory-side cache otherwise (always, for an expert of one row tile).  An expert of few rows is therefore a
+// weight stream at the per-CU HBM rate whatever the kernel does with its rows; the kernel's part is to keep that
+// stream and the large experts' matrix work going side by side on different CUs, and to waste neither.  Measured
+// on full tiles, the copies cost the loop a quarter of its speed even from an L2-hot source: it is their issue
+// (address generation, back-pressure from the L1) in the instruction stream of the waves that feed the matrix core.
 //
 // Row tiles are listed on the device (build_tiles_kernel here, or the permutation
 // kernels inside moe_forward: no host read-back of group sizes); a workgroup's
