@@ -18,7 +18,8 @@
 // Data movement.  A workgroup (8 waves, two per SIMD, one workgroup per CU) owns a
 // work item = (expert, <= 256 activation rows, 256 weight rows) and walks K in
 // steps of 128 through a ring of LDS stages.  Tiles are copied global -> LDS by
-// global_load_lds (no registers in between) ahead of their use.  In
+// global_load_lds (no registers in between) ahead of their use, by one wave of
+// each SIMD (wave set 0); the other (set 1) only computes.  In
 // MODE_GATEUP the 256 weight rows are 128 gate rows + the 128 up rows of the
 // same output columns, so silu(g)*u is lane-local and the 1x128 amax stays
 // inside the workgroup.  Waves form a 4 x 2 grid: wave (wi, xj) owns weight rows
@@ -120,15 +121,17 @@ template <int XF> struct Cls {
   static constexpr int BM = 32 * XF, HALF = BM / 2;
   static constexpr int STAGE_X_OFF = W_TILE_BYTES;
   static constexpr int STAGE_S_OFF = W_TILE_BYTES + BM * BK;
-  // + 256: every wave copies 64 scale slots from its first one on (no lane mask, which would cut the unrolled K
-  // step into blocks); the surplus lanes rewrite the next waves' slots with the same values or land in this pad
+  // + 256: every copying wave copies 64 scale slots from its first one on (no lane mask, which would cut the
+  // unrolled K step into blocks); the surplus lanes rewrite other waves' slots with the same values or land in this pad
   static constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4 + 256;
   static constexpr int NSTAGE = XF >= 5 ? 2 : XF >= 2 ? 3 : 4;
   static constexpr int PRE = NSTAGE - 1;
-  static constexpr int X_GROUPS = 4 * XF;              // 1 KB activation row groups (8 rows) of the tile
-  static constexpr int X_OPS = (X_GROUPS + 7) / 8;     // copies per wave and step; where the groups do not fill the
-                                                       // last round, waves 4-7 repeat the copies of waves 0-3
-  static constexpr int OPS = 4 + X_OPS + 1;            // + 4 weight row groups + 1 scale copy
+  // Only wave set 0 (waves 0-3) issues copies: a copy instruction can hold its wave at the memory pipeline's door
+  // while the L1's queue is full, and with one wave of each SIMD never there the matrix core always has a wave that
+  // can feed it (2-3 % over all eight waves copying).  Wave v copies weight row groups [8v, 8v + 8), activation row
+  // groups v, v + 4, ... and 64 scale slots.
+  static constexpr int X_OPS = XF;                     // activation copies per copying wave and step
+  static constexpr int OPS = 8 + X_OPS + 1;            // + 8 weight row groups + 1 scale copy
   static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
   // copy operations issued after group g: spread over the first SPREAD groups of the step
   static constexpr int SPREAD = XF >= 6 ? XF / 2 : XF >= 3 ? 3 : XF;
@@ -159,14 +162,15 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   const int e = item.expert;
   const int wrow0 = MODE == MODE_GATEUP ? item.col_block * 128 : item.col_block * 256;
 
-  // ---- copy sources (as in grouped_gemm_kernel): wave w fills weight row groups [4w, 4w+4), activation row
-  // groups w, w + 8, ... and 4 XF scale slots
+  // ---- copy sources: copying wave cv (waves 0-3; 4-7 compute the same values and never use them) fills weight row
+  // groups [8 cv, 8 cv + 8), activation row groups cv, cv + 4, ... and 64 scale slots
   const int drow = lane >> 3, dchunk = lane & 7;
-  const uint8_t* wmat = (MODE == MODE_GATEUP && wave >= 4 ? w1 : w0) + (size_t)e * N * K;   // uniform
+  const int cv = wave & 3;
+  const uint8_t* wmat = (MODE == MODE_GATEUP && cv >= 2 ? w1 : w0) + (size_t)e * N * K;   // uniform
   unsigned woff[2];
   {
-    int grow = MODE == MODE_GATEUP ? wrow0 + ((wave * 32) & 127) : wrow0 + wave * 32;
-    if (MODE == MODE_DOWN && grow >= N) grow = N - 32;
+    int grow = MODE == MODE_GATEUP ? wrow0 + ((cv * 64) & 127) : wrow0 + cv * 64;
+    if (MODE == MODE_DOWN && grow >= N) grow = N - 64;   // (a half-full last column block: re-read valid rows)
     const int piece = dchunk ^ (drow >> 1);
     woff[0] = (unsigned)(grow + drow) * (unsigned)K + piece * 16;
     woff[1] = (unsigned)(grow + drow) * (unsigned)K + (piece ^ 4) * 16;
@@ -174,17 +178,17 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   unsigned xoff[C::X_OPS];
 #pragma unroll
   for (int i = 0; i < C::X_OPS; ++i) {
-    int grp = i * NWAVES + wave;
-    if (grp >= C::X_GROUPS) grp -= 4;
+    const int grp = i * 4 + cv;
     const int r = grp * 8 + drow;                              // row within the activation tile
     const int piece = dchunk ^ ((r >> 1) & 7);
     int g = item.row_start + min(r, item.row_count - 1);
     if (row_ids) g = row_ids[g];
     xoff[i] = (unsigned)g * (unsigned)K + piece * 16;
   }
+  const int sbase = BM >= 64 ? min(cv * 64, BM - 64) : 0;   // first of the 64 scale slots this wave copies
   unsigned soff;
   {
-    const int p = min(wave * (BM / 8) + lane, BM - 1);   // slots past the tile land in the pad
+    const int p = min(sbase + lane, BM - 1);   // slots past the tile land in the pad
     const int q = p % HALF;
     const int r = 16 * (2 * (q % XF) + p / HALF) + q / XF;
     int g = item.row_start + min(r, item.row_count - 1);
@@ -194,19 +198,20 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);
   auto issue_op = [&](int kb, int i) {
     const unsigned st = lds0 + (unsigned)(kb % C::NSTAGE) * C::STAGE_BYTES;
-    if (i < 4) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (wave * 4 + i) * 1024u);
-    else if (i < 4 + C::X_OPS) {
-      int grp = (i - 4) * NWAVES + wave;
-      if (grp >= C::X_GROUPS) grp -= 4;
-      dma16(xq + (size_t)kb * BK, xoff[i - 4], st + C::STAGE_X_OFF + grp * 1024u);
-    } else dma4((const uint8_t*)(sx + (size_t)kb * sc.in_kb), soff, st + C::STAGE_S_OFF + wave * (BM / 8) * 4u);
+    if (i < 8) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (cv * 8 + i) * 1024u);
+    else if (i < 8 + C::X_OPS) {
+      const int grp = (i - 8) * 4 + cv;
+      dma16(xq + (size_t)kb * BK, xoff[i - 8], st + C::STAGE_X_OFF + grp * 1024u);
+    } else dma4((const uint8_t*)(sx + (size_t)kb * sc.in_kb), soff, st + C::STAGE_S_OFF + sbase * 4u);
   };
+  if (xj == 0) {
 #pragma unroll
-  for (int s = 0; s < C::PRE; ++s)
-    if (s < KB) {
+    for (int s = 0; s < C::PRE; ++s)
+      if (s < KB) {
 #pragma unroll
-      for (int i = 0; i < C::OPS; ++i) issue_op(s, i);
-    }
+        for (int i = 0; i < C::OPS; ++i) issue_op(s, i);
+      }
+  }
 
   float* wscale = (float*)(lds + CLS_WSCALE_OFF);
   for (int i = tid; i < 2 * KB; i += NT) {
@@ -253,16 +258,20 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   // carries the last ROT activation fragments of a step (and their scales) in registers across the barrier and
   // multiplies them, against the previous step's weights, first thing behind it -- so one wave of each SIMD has
   // matrix work in registers while the other waits for its first fragments from LDS.
-  auto run = [&](auto rot_c) {
+  auto run = [&](auto rot_c, auto issue_c) {
     constexpr int ROT = decltype(rot_c)::value;
+    constexpr bool ISSUE = decltype(issue_c)::value;   // this wave set issues the copies (and waits for them)
     constexpr int NG = XF - ROT;   // groups of the current step done before the next barrier
     constexpr int NH = ROT > 0 ? ROT : 1;
     v8i held[NH];
     float hc0[NH], hc1[NH];
     auto step = [&](int kb, auto first_c, auto copy_c) {
-      constexpr bool FIRST = decltype(first_c)::value, COPY = decltype(copy_c)::value;
+      constexpr bool FIRST = decltype(first_c)::value, COPY = decltype(copy_c)::value && ISSUE;
+      constexpr bool TAIL = !decltype(copy_c)::value;
       // stage kb has landed once only the copies of younger steps are outstanding
-      if (COPY || C::PRE == 1) {
+      if (!ISSUE) {
+        // (the copying waves wait for their copies before the barrier; this set has none in flight)
+      } else if (!TAIL || C::PRE == 1) {
         wait_vm<(C::PRE - 1) * C::OPS>();   // (COPY steps: steps kb+1 .. kb+PRE-1 are in flight)
       } else {
         const int rem = KB - 1 - kb;        // the last steps: fewer and fewer copies are in flight
@@ -378,8 +387,8 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
     for (int f = 0; f < 4; ++f) fm(f, XF - 1, pc0, pc1);
   };
   constexpr int ROT1 = XF > ROTC ? ROTC : XF - 1;   // (fewer groups than that: what there is)
-  if (ROT1 == 0 || xj == 0) run(std::integral_constant<int, 0>{});
-  else run(std::integral_constant<int, ROT1>{});
+  if (xj == 0) run(std::integral_constant<int, 0>{}, std::true_type{});
+  else run(std::integral_constant<int, ROT1>{}, std::false_type{});
   __syncthreads();   // every wave is done reading the ring before the epilogue reuses LDS
 
   // ---- epilogue.  Lane holds, for fragment (f, j): tile row (2j + xj)*16 + fr, weight rows (fragment base) + 4*fq + {0..3}.
