@@ -354,6 +354,18 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
           if (j > 0) fm(f, j - 1, pc0, pc1);
           mm(f, xf[j & 1]);
         }
+        // pinned order: the next group's fragment reads first (a whole group of latency cover), then FMA quadruple f
+        // just before MFMA f (left alone the compiler puts all 16 FMAs before the 4 MFMAs: down GEMM 3-6 % slower)
+        if (j + 1 < NG) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        if (ROT > 0 && j == 0) {
+#pragma unroll
+          for (int i = 0; i < ROT; ++i) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        }
+#pragma unroll
+        for (int f = 0; f < 4; ++f) {
+          if (j > 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
         pc0 = sxv[j] * s0;
         pc1 = sxv[j] * s1;
         if (COPY) {
