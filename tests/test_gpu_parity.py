@@ -376,22 +376,23 @@ def test_graph_replay_matches_eager(jg):
     assert torch.equal(out, want)
 
 
-def test_large_batch_takes_block_major_scales_and_agrees_with_the_debug_path(jg):
+@pytest.mark.parametrize("M,D,E,k,I,SI", [(640, 512, 16, 4, 384, 256), (1100, 384, 8, 2, 128, 0)])
+def test_large_batch_takes_block_major_scales_and_agrees_with_the_debug_path(jg, M, D, E, k, I, SI):
     """Above 2048 routed rows moe_forward hands the GEMMs block-major activation scales, and block-major h scales
     unless the caller asked for the h scales as a debug output (those keep their documented row-major layout).
     Both ways give the same output, bit for bit, and the output holds the plain tolerance against the oracle
     continued from the kernel's own h."""
     import torch
     _say("block-major scales inside moe_forward")
-    prob = H.make_problem(M=640, D=512, E=16, k=4, I=384, SI=256, seed=21, routing="softmax")
-    ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
+    prob = H.make_problem(M=M, D=D, E=E, k=k, I=I, SI=SI, seed=21, routing="softmax")
+    ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"]) if SI else None
     x = H.to_bf16_cuda(prob["x"]); lg = H.to_cuda(prob["logits"])
-    kw = dict(top_k=4, experts=ex, shared=sh)
+    kw = dict(top_k=k, experts=ex, shared=sh)
     plain = jg.moe_experts(x, lg, **kw)                       # no debug outputs: h scales block-major
     out, dbg = jg.moe_experts(x, lg, return_debug=True, **kw)  # h scales row-major in the caller's arrays
     torch.cuda.synchronize()
     assert torch.equal(plain, out)
-    rerun = lambda **h: O.moe_experts(prob["x"], prob["logits"], prob["experts"], top_k=4, shared=prob["shared"], **h)
+    rerun = lambda **h: O.moe_experts(prob["x"], prob["logits"], prob["experts"], top_k=k, shared=prob["shared"], **h)
     H.check_layer_output(out, dbg, rerun(), rerun)
 
 
