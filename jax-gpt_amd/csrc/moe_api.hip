@@ -173,30 +173,20 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
               "forward: unknown routing %d", a->routing);
   int rc;
 
-  // With a shared expert the call forks at once: the side stream quantises the activations and runs the shared
-  // expert, while the caller's stream routes, permutes and lists the work; the routed gate/up GEMM waits for
-  // the quantised activations, the combine for the shared expert's output.  (Event record / wait is also the
-  // pattern a capturing caller's graph turns into forks and joins.)
+  // With a shared expert the call forks: the side stream runs the shared expert while the caller's stream routes,
+  // permutes and runs the routed experts; the combine waits for the shared expert's output.  (Event record / wait
+  // is also the pattern a capturing caller's graph turns into forks and joins.)
+  //   Large batches fork at once: the side stream quantises the activations and starts the shared expert while the
+  // caller's stream routes and permutes; the routed gate/up GEMM waits for the quantised activations.
+  //   Small batches are bound by launch latency, so nothing may stand between the caller's stream and the routed
+  // GEMMs: the activations are quantised on the caller's stream, the side stream waits for them, and the shared
+  // expert's launches are enqueued after the routed ones (they still run beside them: the routed GEMMs take far longer).
+  const bool small_batch = (long long)a->M * a->D <= (1ll << 21);
   hipStream_t side = nullptr;
   hipEvent_t ev_fork = nullptr, ev_quant = nullptr, ev_join = nullptr;
   int rc_shared = MOE_OK;
   bool quant_joined = true;
-  if (a->SI) {
-    if ((rc = side_stream(&side))) return rc;
-    hipError_t e = hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&ev_quant, hipEventDisableTiming);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&ev_join, hipEventDisableTiming);
-    if (e == hipSuccess) e = hipEventRecord(ev_fork, main_s);
-    if (e == hipSuccess) e = hipStreamWaitEvent(side, ev_fork, 0);
-    if (ev_fork) (void)hipEventDestroy(ev_fork);   // released once the recorded work has completed
-    if (e != hipSuccess) {
-      if (ev_quant) (void)hipEventDestroy(ev_quant);
-      if (ev_join) (void)hipEventDestroy(ev_join);
-      return moe_check_hip(e, "forward: fork");
-    }
-    quant_joined = false;
-    rc_shared = quantise(a, b, (moe_stream_t)side);
-    if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
+  auto launch_shared = [&]() {
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
     GemmScales sc = moe_row_major_scales(a->D, a->SI);
     const float* sx_shared = b.sx;
@@ -214,12 +204,42 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
       rc_shared = moe_gemm_down_impl(hsq, shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, ys,
                                      b.gemm_ws_shared, b.gemm_ws_shared_bytes, true,
                                      GemmScales{sc.out_row, sc.out_cb, true, 0, 0}, (moe_stream_t)side);
+  };
+  bool shared_pending = false;
+  if (a->SI) {
+    if ((rc = side_stream(&side))) return rc;
+    hipError_t e = hipEventCreateWithFlags(&ev_quant, hipEventDisableTiming);
+    if (e == hipSuccess) e = hipEventCreateWithFlags(&ev_join, hipEventDisableTiming);
+    if (e == hipSuccess && !small_batch) {
+      e = hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming);
+      if (e == hipSuccess) e = hipEventRecord(ev_fork, main_s);
+      if (e == hipSuccess) e = hipStreamWaitEvent(side, ev_fork, 0);
+      if (ev_fork) (void)hipEventDestroy(ev_fork);   // released once the recorded work has completed
+    }
+    if (e != hipSuccess) {
+      if (ev_quant) (void)hipEventDestroy(ev_quant);
+      if (ev_join) (void)hipEventDestroy(ev_join);
+      return moe_check_hip(e, "forward: fork");
+    }
+    if (small_batch) {
+      rc_shared = quantise(a, b, stream);
+      if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, main_s), "forward: quant event");
+      if (!rc_shared) rc_shared = moe_check_hip(hipStreamWaitEvent(side, ev_quant, 0), "forward: fork");
+      shared_pending = true;
+    } else {
+      quant_joined = false;
+      rc_shared = quantise(a, b, (moe_stream_t)side);
+      if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
+      launch_shared();
+    }
   } else {
     if ((rc = quantise(a, b, stream))) return rc;
   }
   // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
   auto join = [&](int code) {
     if (!a->SI) return code;
+    if (shared_pending && !code && !rc_shared) launch_shared();
+    shared_pending = false;
     hipError_t e1 = hipEventRecord(ev_join, side);
     hipError_t e2 = hipStreamWaitEvent(main_s, ev_join, 0);
     (void)hipEventDestroy(ev_join);
@@ -230,13 +250,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     return moe_check_hip(e2, "forward: join");
   };
 
-  // Small batches: the quantisation is over before the caller's stream has got past the fork, so waiting for it
-  // here costs nothing, and the routed gate/up GEMM then follows the permutation without an event wait between
-  // them (each cross-stream wait costs a few microseconds of launch latency).
-  if (!quant_joined && !rc_shared && (long long)a->M * a->D <= (1ll << 21)) {
-    if ((rc = moe_check_hip(hipStreamWaitEvent(main_s, ev_quant, 0), "forward: quant join"))) return join(rc);
-    quant_joined = true;
-  }
+  if (small_batch && rc_shared) return join(rc_shared);
   // With a router weight the routing kernel adds the matmul's split-K partial sums itself: the (M, E) logits
   // are written only when out_logits asks for them.
   LogitSource src{a->logits, nullptr, 0, a->E, nullptr, nullptr};
