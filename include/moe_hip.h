@@ -208,10 +208,11 @@ typedef struct MoeForwardArgs {
 
 /* Host-side objects moe_forward creates.  No device memory is ever allocated.  With a shared expert (SI > 0) the
  * call (a) creates, on the first such call on a device, ONE side stream for that device (default priority, kept until
- * the process ends, shared by every caller stream and host thread) and (b) creates three hipEvents per call and
- * destroys them before returning (fork, quantised activations ready, shared expert done), so that calls on different
- * streams share no event state.  Consequences: if the caller's stream is being captured into a HIP graph, the side
- * stream joins that capture through the fork event for the length of the call; a second host thread that makes an
+ * the process ends, shared by every caller stream and host thread) and (b) creates two or three hipEvents per call and
+ * destroys them before returning (quantised activations ready, shared expert done, and for large batches a fork
+ * at the call's start), so that calls on different streams share no event state.  Consequences: if the caller's
+ * stream is being captured into a HIP graph, the side stream joins that capture through the first of these events
+ * for the length of the call; a second host thread that makes an
  * eager moe_forward call on the same device while another thread is inside a capturing call would enqueue onto a
  * capturing stream -- that combination is unsupported (serialise such calls, or capture on one thread only).  Without
  * a shared expert no stream or event is created. */
