@@ -338,12 +338,15 @@ def test_reference_entry_points(jg):
     H.assert_close_out(H.bf16_to_np(shared), ref2["shared_out"])
 
 
-def test_graph_replay_matches_eager(jg):
+@pytest.mark.parametrize("M", [64, 4224])
+def test_graph_replay_matches_eager(jg, M):
     """The whole path (side stream for the shared expert included) captured in a HIP graph: every replay, with
-    eager calls and synchronisations between the replays, gives the eager result bit for bit."""
+    eager calls and synchronisations between the replays, gives the eager result bit for bit.  The two batch
+    sizes take the two launch orders of moe_forward: 64 tokens quantise on the caller's stream and enqueue the
+    shared expert after the routed GEMMs, 4224 tokens (more than 2 M activation elements) fork at once."""
     import torch
-    _say("graph replay")
-    prob = H.make_problem(M=64, D=512, E=32, k=4, I=256, SI=256, seed=7, routing="sigmoid_grouped")
+    _say("graph replay", M)
+    prob = H.make_problem(M=M, D=512, E=32, k=4, I=256, SI=256, seed=7, routing="sigmoid_grouped")
     ex = H.experts_to_cuda(prob["experts"]); sh = H.experts_to_cuda(prob["shared"])
     x = H.to_bf16_cuda(prob["x"]); lg = H.to_cuda(prob["logits"])
     kw = dict(top_k=4, experts=ex, shared=sh, routing="sigmoid_grouped", n_group=4, topk_group=2)
