@@ -40,13 +40,25 @@ inline int moe_raise_lds_limit(const void* kernel, int bytes, std::atomic<unsign
 // depends on the group sizes and the tile height only, so the gate/up and the down GEMM of a layer share it.
 struct TileHeader {
   int n_tiles;
-  int pad[3];
-  // Where the work of XCD k begins, as a tile position with 20 fraction bits (xcd_q[0] = 0, xcd_q[8] = n_tiles << 20);
+  // The first n_static tiles are dealt to the XCDs in fixed shares (xcd_q).  The rest -- the smallest experts, last in
+  // the list -- are a pool that the workgroups of every XCD draw from once their share is done, an item at a time
+  // through pool_next (one counter per GEMM of the layer: gate/up, down; the list's builder sets them to zero, so a
+  // list serves one launch of each).  An XCD that is ahead takes more of the pool: it evens out what the fixed
+  // shares cannot know (the XCDs' paces differ by a few per cent, and so does the cost estimate behind the shares).
+  int n_static;
+  int pool_next[2];
+  // Where the work of XCD k begins, as a tile position with 20 fraction bits (xcd_q[0] = 0, xcd_q[8] = n_static << 20);
   // a GEMM with ncb column blocks per row tile gives XCD k the items [xcd_q[k] * ncb >> 20, xcd_q[k + 1] * ncb >> 20).
   long long xcd_q[9];
   long long pad2;
 };
 constexpr int kTileQBits = 20;
+// The pool holds at most max_tiles / 16 tiles, and an XCD may draw up to twice its eighth of it: the grouped GEMM
+// launches this many workgroups per XCD beyond its fixed share for a GEMM of ncb column blocks per row tile.
+constexpr int kPoolShift = 4;    // (a pool of max_tiles / 8 and up to 4 or 6 tail rounds measured 0.5-1 % slower)
+constexpr int kTailRounds = 3;   // rounds of the ranking (8 experts each) that end a bin or go to the pool
+__host__ __device__ inline int moe_pool_tile_limit(int max_tiles) { return max_tiles >> kPoolShift; }
+__host__ __device__ inline int moe_pool_workgroups(long long pool_items) { return (int)(pool_items >> 2) + 1; }
 // The grouped GEMM launches ceil(max_tiles * ncb / 8) + 2 workgroups per XCD: a split whose largest share stays
 // within max_tiles / 8 tiles fits whatever ncb is (max_tiles is a worst case over all group sizes, so a real list
 // is usually a good deal shorter and its shares fit with room to spare).
@@ -93,53 +105,77 @@ __host__ __device__ inline void moe_tile_span(int rows, int nt, int t, int& star
 // GEMM), and equal counts left the XCD with the tallest tiles some 3 % more work than the average.  All tiles of an
 // expert cost alike, so a cut inside an expert sits at the same fraction of its items as of its cost.
 __device__ inline int moe_tile_cost(int rows) { return 8 * moe_tile_count(rows) + ((rows + 31) >> 5); }   // (< 2^31 for 2^32 / 128 rows)
-__device__ inline void moe_tile_even_shares(TileHeader* hdr, int n_tiles) {   // one thread
+__device__ inline void moe_tile_even_shares(TileHeader* hdr, int n_static, int n_tiles) {   // one thread
   hdr->n_tiles = n_tiles;
-  for (int k = 0; k <= 8; ++k) hdr->xcd_q[k] = (((long long)n_tiles << kTileQBits) * k) >> 3;
+  hdr->n_static = n_static;
+  hdr->pool_next[0] = hdr->pool_next[1] = 0;
+  for (int k = 0; k <= 8; ++k) hdr->xcd_q[k] = (((long long)n_static << kTileQBits) * k) >> 3;
 }
 __device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int* lds_key, int* total_tiles,
                                      TileHeader* hdr, int max_tiles) {
   __shared__ long long cut_q[9];
+  __shared__ int tail_tiles[kTailRounds];   // tiles of the last, last but one, ... round of the ranking
   lds_rows[e] = e < E ? rows : 0;
+  if (e < kTailRounds) tail_tiles[e] = 0;
   __syncthreads();
   int key = e;
+  int rank = 0, nz = 0;
   if (e < E) {
-    int rank = 0, nz = 0;
 #pragma unroll 8
     for (int o = 0; o < E; ++o) {
       const int r = lds_rows[o];
       rank += (r > rows || (r == rows && o < e)) ? 1 : 0;
       nz += r > 0 ? 1 : 0;
     }
-    const int round = rank >> 3, posn = rank & 7;
+  }
+  const int nr = (nz + 7) >> 3;   // rounds that hold a non-empty expert
+  const int tail = nr / 4 < kTailRounds ? nr / 4 : kTailRounds;   // (3 rounds = 24 experts over the 8 bins; 6 measured no better)
+  const int round = rank >> 3;
+  if (e < E && rows > 0 && round >= nr - tail) atomicAdd(&tail_tiles[nr - 1 - round], moe_tile_count(rows));
+  __syncthreads();
+  // The pool: as many of the tail rounds, from the last one, as fit the launch's spare workgroups.
+  int pooled = 0;
+  for (int t = 0, sum = 0; e < E && t < tail; ++t) {
+    sum += tail_tiles[t];
+    if (sum > moe_pool_tile_limit(max_tiles)) break;
+    pooled = t + 1;
+  }
+  if (e < E && rows > 0 && round >= nr - pooled) {
+    key = 1024 + rank;   // behind every bin (keys below 1024), the tallest of the pool first
+  } else if (e < E) {
+    const int posn = rank & 7;
     // Inside a bin the experts alternate between the large and the small end of the ranking (largest, smallest,
     // second largest, ...): tall tiles are matrix work on lines that mostly hit L2, short tiles are weight streams
     // from HBM, and a launch that runs them side by side from start to end keeps both busy and its power draw even
     // (largest first throughout: 1.4 % slower on the heavy-tailed DeepSeek-V3 routing, 4 % on the Qwen3-MoE case).
-    // The smallest experts of a bin stay at its end: the launch ends with its shortest items.
-    const int nr = (nz + 7) >> 3;   // rounds that hold a non-empty expert
-    const int tail = nr / 4 < 3 ? nr / 4 : 3;   // (3 rounds = 24 experts over the 8 bins; 6 measured no better)
+    // The smallest experts of a bin stay at its end (those that the pool does not take): the launch ends with its
+    // shortest items.
     const int mixed = nr - tail;
     const int pos = round >= mixed ? round : (round < (mixed + 1) / 2 ? 2 * round : 2 * (mixed - 1 - round) + 1);
     key = ((round & 1) ? 7 - posn : posn) * 128 + pos;   // E <= 1024: at most 128 rounds
   }
   lds_key[e] = key;
   __syncthreads();
-  int first = 0, total = 0;
+  int first = 0, total = 0, n_static = 0;
   int cost_before = 0, cost_all = 0;
+  if (e < E) {   // (the threads past the last expert only keep the barriers company)
 #pragma unroll 8
-  for (int o = 0; o < E; ++o) {
-    const int t = moe_tile_count(lds_rows[o]);
-    const int c = 8 * t + ((lds_rows[o] + 31) >> 5);
-    const bool before = lds_key[o] < key;
-    total += t;
-    cost_all += c;
-    first += before ? t : 0;
-    cost_before += before ? c : 0;
+    for (int o = 0; o < E; ++o) {
+      const int t = moe_tile_count(lds_rows[o]);
+      const bool fixed = lds_key[o] < 1024;   // (not in the pool)
+      const int c = fixed ? 8 * t + ((lds_rows[o] + 31) >> 5) : 0;
+      const bool before = lds_key[o] < key;
+      total += t;
+      n_static += fixed ? t : 0;
+      cost_all += c;
+      first += before ? t : 0;
+      cost_before += before ? c : 0;
+    }
   }
-  *total_tiles = total;
-  // cut k sits where the cost reaches k/8 of the whole: inside exactly one expert, whose thread places it
-  if (e < E && rows > 0) {
+  *total_tiles = total;   // (valid for e < E)
+  // cut k sits where the cost of the fixed shares reaches k/8 of their whole: inside exactly one expert, whose
+  // thread places it
+  if (e < E && rows > 0 && key < 1024) {
     const long long mine = moe_tile_cost(rows);
     const int nt = moe_tile_count(rows);
     for (int k = 1; k < 8; ++k) {
@@ -152,16 +188,14 @@ __device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int*
   __syncthreads();
   if (e == 0) {
     const int n = total < max_tiles ? total : max_tiles;
+    const int ns = n_static < n ? n_static : n;
     cut_q[0] = 0;
-    cut_q[8] = (long long)n << kTileQBits;
-    bool fits = total > 0 && total <= max_tiles;
+    cut_q[8] = (long long)ns << kTileQBits;
+    bool fits = ns > 0 && total <= max_tiles;
     for (int k = 0; k < 8 && fits; ++k) fits = cut_q[k + 1] - cut_q[k] <= moe_xcd_share_cap_q(max_tiles);
-    if (fits) {
-      hdr->n_tiles = n;
+    moe_tile_even_shares(hdr, ns, n);   // (a share beyond what the launch provides workgroups for: equal counts always fit)
+    if (fits)
       for (int k = 0; k <= 8; ++k) hdr->xcd_q[k] = cut_q[k];
-    } else {
-      moe_tile_even_shares(hdr, n);   // (a share beyond what the launch provides workgroups for: equal counts always fit)
-    }
   }
   return first;
 }

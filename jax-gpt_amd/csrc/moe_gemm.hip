@@ -497,8 +497,22 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
   // contiguous ranges of about equal cost (workgroup ids are issued round-robin over XCDs)
   const int ncb = MODE == MODE_GATEUP ? N / 128 : (N + 255) / 256;
   const int xcd = blockIdx.x & 7;
-  const int item_id = (int)((hdr->xcd_q[xcd] * ncb) >> kTileQBits) + (int)(blockIdx.x >> 3);
-  if (item_id >= (int)((hdr->xcd_q[xcd + 1] * ncb) >> kTileQBits)) return;
+  int item_id = (int)((hdr->xcd_q[xcd] * ncb) >> kTileQBits) + (int)(blockIdx.x >> 3);
+  const int share_end = (int)((hdr->xcd_q[xcd + 1] * ncb) >> kTileQBits);
+  if (item_id >= share_end) {
+    // behind the XCD's fixed share: the pool of the smallest experts' items, drawn one at a time by whoever gets
+    // there (TileHeader); an XCD may draw up to twice its eighth of it
+    const int pool_first = hdr->n_static * ncb;
+    const int pool_items = (hdr->n_tiles - hdr->n_static) * ncb;
+    if (pool_items == 0 || item_id - share_end >= moe_pool_workgroups(pool_items)) return;   // (uniform: the whole workgroup leaves)
+    int* slot = (int*)lds;
+    if (threadIdx.x == 0) *slot = atomicAdd(const_cast<int*>(&hdr->pool_next[MODE]), 1);
+    __syncthreads();
+    const int drawn = *slot;
+    __syncthreads();   // (the work item's first copies overwrite the slot)
+    if (drawn >= pool_items) return;
+    item_id = pool_first + drawn;
+  }
   Item item;
   {
     const TileEntry te = tiles[item_id / ncb];   // entries [first_tile, first_tile + tiles) all describe this expert
@@ -576,8 +590,10 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
   if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE>, CLS_LDS_BYTES, lds_raised)) return rc;
   const long long max_items = (long long)l.max_tiles * col_blocks(MODE, N);
   MOE_REQUIRE(max_items < (1ll << 30), MOE_ERR_BAD_SHAPE, "gemm: %lld work items exceed the grid limit", max_items);
-  // sized by the worst case of the largest XCD share (moe_xcd_share_cap_q); surplus workgroups exit at once
-  const int grid = 8 * (int)((max_items + 7) / 8 + 2);
+  // sized by the worst case of the largest XCD share (moe_xcd_share_cap_q) and of an XCD's draws from the pool;
+  // surplus workgroups exit at once
+  const long long pool_max = (long long)moe_pool_tile_limit(l.max_tiles) * col_blocks(MODE, N);
+  const int grid = 8 * (int)((max_items + 7) / 8 + 2 + moe_pool_workgroups(pool_max));
   hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NT), CLS_LDS_BYTES, s, xq, sx, row_ids, w0, sw0, w1,
                      sw1, l.hdr, l.tiles, K, N, out, out_scale, sc);
   return moe_check_hip(hipGetLastError(), "gemm launch");
