@@ -43,7 +43,11 @@
 // work item is a (row tile, column block) pair derived from its index, in
 // [expert][column block][row tile] order, and the items are dealt to the 8 XCDs in
 // contiguous ranges, so the row tiles and column blocks that share a weight slab
-// or an activation tile run together under one L2.
+// or an activation tile run together under one L2.  The items of the smallest
+// experts (weight streams, nothing to share) are not dealt out: they sit behind
+// the eight ranges as a pool from which the workgroups that follow an XCD's range
+// draw one item each through a counter (TileHeader), so an XCD that is ahead
+// takes more of them.
 #include <stdlib.h>
 
 #include <mutex>
