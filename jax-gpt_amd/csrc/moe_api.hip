@@ -113,9 +113,11 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool r
 
 namespace {
 // the activations the layer computes from: x itself, or its RMS-normalised form (kept in bf16 for the router)
-int quantise(const MoeForwardArgs* a, const ForwardBuffers& b, moe_stream_t stream) {
-  if (a->norm_weight) return moe_rmsnorm_quant(a->x, a->norm_weight, a->norm_eps, a->M, a->D, b.normed, b.xq, b.sx, stream);
-  return moe_quant_act(a->x, a->M, a->D, b.xq, b.sx, stream);
+// (sx_blocked: an optional second copy of the scales, block-major in token order, for the shared expert of a large batch)
+int quantise(const MoeForwardArgs* a, const ForwardBuffers& b, float* sx_blocked, moe_stream_t stream) {
+  if (a->norm_weight)
+    return moe_rmsnorm_quant_impl(a->x, a->norm_weight, a->norm_eps, a->M, a->D, b.normed, b.xq, b.sx, sx_blocked, stream);
+  return moe_quant_act_impl(a->x, a->M, a->D, b.xq, b.sx, sx_blocked, stream);
 }
 }  // namespace
 
@@ -186,19 +188,24 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   hipEvent_t ev_fork = nullptr, ev_quant = nullptr, ev_join = nullptr;
   int rc_shared = MOE_OK;
   bool quant_joined = true;
-  auto launch_shared = [&]() {
+  // the shared expert's one group and its tile list (they depend on M alone: enqueued ahead of the quantiser where
+  // the side stream runs it, so that nothing stands between the quantiser and the shared gate/up GEMM)
+  auto list_shared = [&]() {
     hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
+    if (!rc_shared)
+      rc_shared = moe_gemm_build_tile_list(b.dense_off, 1, a->M, b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
+  };
+  auto launch_shared = [&]() {
     GemmScales sc = moe_row_major_scales(a->D, a->SI);
     const float* sx_shared = b.sx;
-    if (blocked_scales) {
-      if (!rc_shared) rc_shared = moe_gather_scales(b.sx, nullptr, a->M, a->D / 128, b.sx_blocked, (moe_stream_t)side);
+    if (blocked_scales) {   // (block-major scales in token order: written by the quantiser itself)
       sx_shared = b.sx_blocked;
       sc.in_row = 1, sc.in_kb = a->M, sc.in_listed = true;
       if (!a->out_shs) sc.out_row = 1, sc.out_cb = a->M;   // (a debug copy of the h scales keeps the documented layout)
     }
     if (!rc_shared)
       rc_shared = moe_gemm_gateup_impl(b.xq, sx_shared, nullptr, a->ws_gate, a->sws_gate, a->ws_up, a->sws_up, b.dense_off,
-                                       1, a->M, a->D, a->SI, hsq, shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, false, sc,
+                                       1, a->M, a->D, a->SI, hsq, shs, b.gemm_ws_shared, b.gemm_ws_shared_bytes, true, sc,
                                        (moe_stream_t)side);
     if (!rc_shared)   // same rows, same tile height: the list the gate/up launch built serves the down launch too
       rc_shared = moe_gemm_down_impl(hsq, shs, a->ws_down, a->sws_down, b.dense_off, 1, a->M, a->SI, a->D, ys,
@@ -222,23 +229,27 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
       return moe_check_hip(e, "forward: fork");
     }
     if (small_batch) {
-      rc_shared = quantise(a, b, stream);
+      rc_shared = quantise(a, b, blocked_scales ? b.sx_blocked : nullptr, stream);
       if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, main_s), "forward: quant event");
       if (!rc_shared) rc_shared = moe_check_hip(hipStreamWaitEvent(side, ev_quant, 0), "forward: fork");
       shared_pending = true;
     } else {
       quant_joined = false;
-      rc_shared = quantise(a, b, (moe_stream_t)side);
+      list_shared();
+      if (!rc_shared) rc_shared = quantise(a, b, blocked_scales ? b.sx_blocked : nullptr, (moe_stream_t)side);
       if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
       launch_shared();
     }
   } else {
-    if ((rc = quantise(a, b, stream))) return rc;
+    if ((rc = quantise(a, b, nullptr, stream))) return rc;
   }
   // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
   auto join = [&](int code) {
     if (!a->SI) return code;
-    if (shared_pending && !code && !rc_shared) launch_shared();
+    if (shared_pending && !code && !rc_shared) {
+      list_shared();
+      launch_shared();
+    }
     shared_pending = false;
     hipError_t e1 = hipEventRecord(ev_join, side);
     hipError_t e2 = hipStreamWaitEvent(main_s, ev_join, 0);

@@ -223,6 +223,12 @@ int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, in
 // own.  moe_gemm_tile_list describes the list the GEMMs of (R rows, E experts) expect in ws, so that the permutation
 // kernels, which hold every expert's row range anyway, can write it (moe_permute_impl) and no launch is spent on it.
 int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list);
+int moe_gemm_build_tile_list(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream);
+// the activation quantisers with an optional second copy of the scales, block-major in row order ((K/128, R): what
+// GemmScales{1, R} reads) -- spares the shared expert of a large batch the separate transposition
+int moe_quant_act_impl(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream);
+int moe_rmsnorm_quant_impl(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
+                           uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream);
 int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_sizes, int32_t* group_offsets,
                      int32_t* sorted_token_ids, int32_t* sort_order, int32_t* inv_perm, void* ws, size_t ws_bytes,
                      TileList tiles, moe_stream_t stream);

@@ -724,6 +724,15 @@ extern "C" int moe_gemm_down_fp8_layout(const uint8_t* hq, const float* sh, cons
   return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, sc, stream);
 }
 
+// Builds, ahead of the GEMM launches, the list that they read from ws when they are told list_built = true.
+int moe_gemm_build_tile_list(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream) {
+  TileList l;
+  if (int rc = moe_gemm_tile_list(R, E, ws, ws_bytes, &l)) return rc;
+  MOE_REQUIRE(group_offsets, MOE_ERR_NULL, "gemm tiles: null group offsets");
+  hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, l);
+  return moe_check_hip(hipGetLastError(), "gemm tiles launch");
+}
+
 // The tile list that the GEMM launches of (R rows, E experts) read from ws when they are told list_built = true.
 int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list) {
   MOE_REQUIRE(ws && list, MOE_ERR_NULL, "gemm tiles: null pointer");

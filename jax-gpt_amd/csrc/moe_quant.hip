@@ -13,7 +13,8 @@ struct alignas(16) bf16x8 { bf16_t v[8]; };
 // 16 lanes per 128-wide group, 8 bf16 (16 B) per lane
 __global__ __launch_bounds__(256) void quant_act_kernel(const bf16x8* __restrict__ x, long long n_pieces,
                                                        int groups_per_row, uint2* __restrict__ xq,
-                                                       float* __restrict__ sx) {
+                                                       float* __restrict__ sx, float* __restrict__ sx_blocked,
+                                                       int R) {
   long long p = (long long)blockIdx.x * 256 + threadIdx.x;
   bool ok = p < n_pieces;
   bf16x8 in = {};
@@ -33,7 +34,14 @@ __global__ __launch_bounds__(256) void quant_act_kernel(const bf16x8* __restrict
     out.x = pack4_e4m3(f[0] * scale, f[1] * scale, f[2] * scale, f[3] * scale);
     out.y = pack4_e4m3(f[4] * scale, f[5] * scale, f[6] * scale, f[7] * scale);
     xq[p] = out;
-    if ((threadIdx.x & 15) == 0) sx[p >> 4] = scale_inv;
+    if ((threadIdx.x & 15) == 0) {
+      const long long g = p >> 4;
+      sx[g] = scale_inv;
+      if (sx_blocked) {   // the same scale in the (K/128, R) array
+        const int row = (int)(g / groups_per_row), kb = (int)(g - (long long)row * groups_per_row);
+        sx_blocked[(size_t)kb * R + row] = scale_inv;
+      }
+    }
   }
 }
 
@@ -47,7 +55,8 @@ constexpr int kNormPieces = 4;   // D <= 256 * 8 * 4 = 8192
 
 __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const bf16x8* __restrict__ x, const float* __restrict__ weight,
                                                            float eps, int D, bf16x8* __restrict__ normed,
-                                                           uint2* __restrict__ xq, float* __restrict__ sx) {
+                                                           uint2* __restrict__ xq, float* __restrict__ sx,
+                                                           float* __restrict__ sx_blocked) {
   __shared__ float wave_sum[4];
   const int row = blockIdx.x, P = D / 8, t = threadIdx.x;
   const bf16x8* xr = x + (size_t)row * P;
@@ -94,7 +103,10 @@ __global__ __launch_bounds__(256) void rmsnorm_quant_kernel(const bf16x8* __rest
       out.x = pack4_e4m3(f[i][0] * scale, f[i][1] * scale, f[i][2] * scale, f[i][3] * scale);
       out.y = pack4_e4m3(f[i][4] * scale, f[i][5] * scale, f[i][6] * scale, f[i][7] * scale);
       xq[(size_t)row * P + p] = out;
-      if ((t & 15) == 0) sx[((size_t)row * P + p) >> 4] = scale_inv;
+      if ((t & 15) == 0) {
+        sx[((size_t)row * P + p) >> 4] = scale_inv;
+        if (sx_blocked) sx_blocked[(size_t)(p >> 4) * gridDim.x + row] = scale_inv;   // the (K/128, M) array
+      }
     }
   }
 }
@@ -133,6 +145,9 @@ __global__ __launch_bounds__(256) void quant_weight_kernel(const T* __restrict__
 }  // namespace
 
 extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream) {
+  return moe_quant_act_impl(x_bf16, R, K, xq, sx, nullptr, stream);
+}
+int moe_quant_act_impl(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream) {
   MOE_REQUIRE(R == 0 || (x_bf16 && xq && sx), MOE_ERR_NULL, "quant_act: null pointer");
   MOE_REQUIRE(R >= 0 && K > 0 && K % MOE_QBLOCK == 0, MOE_ERR_BAD_SHAPE, "quant_act: K=%d must be a positive multiple of 128 (R=%d)", K, R);
   MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(xq), MOE_ERR_BAD_ALIGN, "quant_act: pointers must be 16-byte aligned");
@@ -141,12 +156,16 @@ extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, floa
   long long blocks = (pieces + 255) / 256;
   MOE_REQUIRE(blocks < (1ll << 31), MOE_ERR_BAD_SHAPE, "quant_act: too many elements");
   hipLaunchKernelGGL(quant_act_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16x8*)x_bf16, pieces, K / 128, (uint2*)xq, sx);
+                     (const bf16x8*)x_bf16, pieces, K / 128, (uint2*)xq, sx, sx_blocked, R);
   return moe_check_hip(hipGetLastError(), "quant_act launch");
 }
 
 extern "C" int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
                                  uint8_t* xq, float* sx, moe_stream_t stream) {
+  return moe_rmsnorm_quant_impl(x_bf16, weight, eps, M, D, normed_bf16, xq, sx, nullptr, stream);
+}
+int moe_rmsnorm_quant_impl(const void* x_bf16, const float* weight, float eps, int M, int D, void* normed_bf16,
+                           uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream) {
   MOE_REQUIRE((M == 0 || (x_bf16 && xq && sx)) && weight, MOE_ERR_NULL, "rmsnorm_quant: null pointer");
   MOE_REQUIRE(M >= 0 && D > 0 && D % MOE_QBLOCK == 0 && D <= 256 * 8 * kNormPieces, MOE_ERR_BAD_SHAPE,
               "rmsnorm_quant: D=%d must be a multiple of 128, at most %d (M=%d)", D, 256 * 8 * kNormPieces, M);
@@ -154,7 +173,7 @@ extern "C" int moe_rmsnorm_quant(const void* x_bf16, const float* weight, float 
               "rmsnorm_quant: pointers must be 16-byte aligned");
   if (M == 0) return MOE_OK;
   hipLaunchKernelGGL(rmsnorm_quant_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, (const bf16x8*)x_bf16, weight, eps,
-                     D, (bf16x8*)normed_bf16, (uint2*)xq, sx);
+                     D, (bf16x8*)normed_bf16, (uint2*)xq, sx, sx_blocked);
   return moe_check_hip(hipGetLastError(), "rmsnorm_quant launch");
 }
 
