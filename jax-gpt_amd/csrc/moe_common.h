@@ -241,6 +241,7 @@ struct GemmScales {
   int in_row, in_kb;
   bool in_listed;
   int out_row, out_cb;   // gate/up only: scale of (row, column block cb) of h = sh[row * out_row + cb * out_cb]
+  bool stream_out;       // down only, set by the launch: y is stored with non-temporal stores
 };
 inline GemmScales moe_row_major_scales(int K, int I) { return GemmScales{K / 128, 1, false, I / 128, 1}; }
 int moe_gemm_gateup_impl(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uint8_t* w_gate,
