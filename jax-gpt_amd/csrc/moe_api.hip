@@ -213,6 +213,14 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
                                      GemmScales{sc.out_row, sc.out_cb, true, 0, 0}, (moe_stream_t)side);
   };
   bool shared_pending = false;
+  // Where the quantiser would run on the caller's stream just ahead of the routing kernel, the routing launch
+  // carries its blocks instead (QuantJob: the two are independent; one launch less and they overlap).  Not with
+  // an RMSNorm in front: the router then reads what the quantiser writes.
+  const bool quant_in_route = (!a->SI || small_batch) && !a->norm_weight && a->M > 0;
+  QuantJob quant_job{};
+  if (quant_in_route &&
+      (rc = moe_quant_act_job(a->x, a->M, a->D, b.xq, b.sx, (a->SI && blocked_scales) ? b.sx_blocked : nullptr, &quant_job)))
+    return rc;
   if (a->SI) {
     if ((rc = side_stream(&side))) return rc;
     hipError_t e = hipEventCreateWithFlags(&ev_quant, hipEventDisableTiming);
@@ -229,9 +237,11 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
       return moe_check_hip(e, "forward: fork");
     }
     if (small_batch) {
-      rc_shared = quantise(a, b, blocked_scales ? b.sx_blocked : nullptr, stream);
-      if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, main_s), "forward: quant event");
-      if (!rc_shared) rc_shared = moe_check_hip(hipStreamWaitEvent(side, ev_quant, 0), "forward: fork");
+      if (!quant_in_route) {
+        rc_shared = quantise(a, b, blocked_scales ? b.sx_blocked : nullptr, stream);
+        if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, main_s), "forward: quant event");
+        if (!rc_shared) rc_shared = moe_check_hip(hipStreamWaitEvent(side, ev_quant, 0), "forward: fork");
+      }   // (else: the same record and wait follow the routing launch, below)
       shared_pending = true;
     } else {
       quant_joined = false;
@@ -240,7 +250,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
       if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, side), "forward: quant event");
       launch_shared();
     }
-  } else {
+  } else if (!quant_in_route) {
     if ((rc = quantise(a, b, nullptr, stream))) return rc;
   }
   // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
@@ -281,12 +291,18 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     if (a->w_shared_gate) shared_gate = gate_out;
     src = LogitSource{nullptr, (const float*)b.router_ws, splits, n_cols, a->out_logits, gate_out};
   }
+  const QuantJob* carried = quant_in_route ? &quant_job : nullptr;
   if (a->routing == MOE_ROUTING_SOFTMAX)
-    rc = moe_route_softmax_impl(src, a->M, a->E, a->k, a->renorm, idx, w, stream);
+    rc = moe_route_softmax_impl(src, a->M, a->E, a->k, a->renorm, idx, w, stream, carried);
   else
     rc = moe_route_sigmoid_grouped_impl(src, a->bias, a->M, a->E, a->n_group, a->topk_group, a->k, a->renorm,
-                                        a->routed_scale, idx, w, stream);
+                                        a->routed_scale, idx, w, stream, carried);
   if (rc) return join(rc);
+  if (quant_in_route && a->SI) {   // the side stream's shared expert waits for the activations quantised above
+    hipError_t e = hipEventRecord(ev_quant, main_s);
+    if (e == hipSuccess) e = hipStreamWaitEvent(side, ev_quant, 0);
+    if (e != hipSuccess) return join(moe_check_hip(e, "forward: quant event"));
+  }
   // the permutation kernels also list the routed GEMMs' row tiles (they hold every expert's row range anyway)
   TileList tiles;
   if ((rc = moe_gemm_tile_list(R, a->E, b.gemm_ws, b.gemm_ws_bytes, &tiles))) return join(rc);

@@ -214,11 +214,24 @@ struct LogitSource {
 int moe_router_partials(const void* x_bf16, int M, int D, const void* w_router_bf16, int E,
                         const void* w_shared_gate_bf16, void* ws, size_t ws_bytes, int* splits_used, int* n_cols,
                         moe_stream_t stream);
+// An activation quantisation that a routing launch carries along (moe_quant_device.h): `blocks` blocks of 256
+// 16-byte pieces behind the routing kernel's own blocks.  blocks == 0: none.
+struct QuantJob {
+  const void* x;        // (R, K) bf16
+  long long n_pieces;   // R * K / 8
+  int groups_per_row;   // K / 128
+  int R;
+  uint8_t* xq;
+  float* sx;
+  float* sx_blocked;    // optional (K/128, R) copy of the scales
+  unsigned blocks;
+};
+int moe_quant_act_job(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, QuantJob* job);
 int moe_route_softmax_impl(const LogitSource& src, int M, int E, int k, int renorm, int32_t* idx, float* w,
-                           moe_stream_t stream);
+                           moe_stream_t stream, const QuantJob* quant = nullptr);
 int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, int M, int E, int n_group,
                                    int topk_group, int k, int renorm, float routed_scale, int32_t* idx, float* w,
-                                   moe_stream_t stream);
+                                   moe_stream_t stream, const QuantJob* quant = nullptr);
 // grouped GEMMs with an optional pre-built tile list in ws (moe_gemm.hip); the extern "C" entry points build their
 // own.  moe_gemm_tile_list describes the list the GEMMs of (R rows, E experts) expect in ws, so that the permutation
 // kernels, which hold every expert's row range anyway, can write it (moe_permute_impl) and no launch is spent on it.

@@ -5,45 +5,13 @@
 // jax_gpt/models/qwen35/fp8.py:30-45).  Weights: 128x128 blocks in the
 // (E, out, in) layout of quantize.py:31-42.
 #include "moe_common.h"
+#include "moe_quant_device.h"
 
 namespace {
 
-struct alignas(16) bf16x8 { bf16_t v[8]; };
+typedef moe_bf16x8 bf16x8;
 
-// 16 lanes per 128-wide group, 8 bf16 (16 B) per lane
-__global__ __launch_bounds__(256) void quant_act_kernel(const bf16x8* __restrict__ x, long long n_pieces,
-                                                       int groups_per_row, uint2* __restrict__ xq,
-                                                       float* __restrict__ sx, float* __restrict__ sx_blocked,
-                                                       int R) {
-  long long p = (long long)blockIdx.x * 256 + threadIdx.x;
-  bool ok = p < n_pieces;
-  bf16x8 in = {};
-  if (ok) in = x[p];
-  float f[8], amax = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    f[i] = bf16_to_f32(in.v[i]);
-    amax = fmaxf(amax, fabsf(f[i]));
-  }
-#pragma unroll
-  for (int off = 1; off < 16; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, MOE_WAVE));
-  float scale, scale_inv;
-  fp8_scales(amax, scale, scale_inv);
-  if (ok) {
-    uint2 out;
-    out.x = pack4_e4m3(f[0] * scale, f[1] * scale, f[2] * scale, f[3] * scale);
-    out.y = pack4_e4m3(f[4] * scale, f[5] * scale, f[6] * scale, f[7] * scale);
-    xq[p] = out;
-    if ((threadIdx.x & 15) == 0) {
-      const long long g = p >> 4;
-      sx[g] = scale_inv;
-      if (sx_blocked) {   // the same scale in the (K/128, R) array
-        const int row = (int)(g / groups_per_row), kb = (int)(g - (long long)row * groups_per_row);
-        sx_blocked[(size_t)kb * R + row] = scale_inv;
-      }
-    }
-  }
-}
+__global__ __launch_bounds__(256) void quant_act_kernel(const QuantJob q) { moe_quant_act_block(q, blockIdx.x); }
 
 // RMSNorm fused with the activation quantiser: one workgroup per row, the row stays in registers between the
 // two passes.  normed = bf16((x / sqrt(mean(x^2) + eps)) * (1 + weight)), the Qwen3.5 convention of
@@ -147,16 +115,22 @@ __global__ __launch_bounds__(256) void quant_weight_kernel(const T* __restrict__
 extern "C" int moe_quant_act(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, moe_stream_t stream) {
   return moe_quant_act_impl(x_bf16, R, K, xq, sx, nullptr, stream);
 }
-int moe_quant_act_impl(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream) {
+// checks the arguments of an activation quantisation and describes it (for its own launch, or a routing launch's)
+int moe_quant_act_job(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, QuantJob* job) {
   MOE_REQUIRE(R == 0 || (x_bf16 && xq && sx), MOE_ERR_NULL, "quant_act: null pointer");
   MOE_REQUIRE(R >= 0 && K > 0 && K % MOE_QBLOCK == 0, MOE_ERR_BAD_SHAPE, "quant_act: K=%d must be a positive multiple of 128 (R=%d)", K, R);
   MOE_REQUIRE(MOE_ALIGNED16(x_bf16) && MOE_ALIGNED16(xq), MOE_ERR_BAD_ALIGN, "quant_act: pointers must be 16-byte aligned");
-  if (R == 0) return MOE_OK;
-  long long pieces = (long long)R * K / 8;
-  long long blocks = (pieces + 255) / 256;
+  const long long pieces = (long long)R * K / 8;
+  const long long blocks = (pieces + 255) / 256;
   MOE_REQUIRE(blocks < (1ll << 31), MOE_ERR_BAD_SHAPE, "quant_act: too many elements");
-  hipLaunchKernelGGL(quant_act_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const bf16x8*)x_bf16, pieces, K / 128, (uint2*)xq, sx, sx_blocked, R);
+  *job = QuantJob{x_bf16, pieces, K / 128, R, xq, sx, sx_blocked, (unsigned)blocks};
+  return MOE_OK;
+}
+int moe_quant_act_impl(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream) {
+  QuantJob job;
+  if (int rc = moe_quant_act_job(x_bf16, R, K, xq, sx, sx_blocked, &job)) return rc;
+  if (R == 0) return MOE_OK;
+  hipLaunchKernelGGL(quant_act_kernel, dim3(job.blocks), dim3(256), 0, (hipStream_t)stream, job);
   return moe_check_hip(hipGetLastError(), "quant_act launch");
 }
 

@@ -9,6 +9,7 @@
 //
 // Replaces jax_gpt/models/qwen35/moe.py:51-53 (softmax, lax.top_k, renormalise).
 #include "moe_common.h"
+#include "moe_quant_device.h"
 
 namespace {
 
@@ -90,7 +91,12 @@ __device__ __forceinline__ void finish_shared_gate(const LogitSource& src, int M
 template <int VPL>
 __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_softmax_kernel(
     const LogitSource src, int M, int E, int k, int renorm, int32_t* __restrict__ idx,
-    float* __restrict__ w) {
+    float* __restrict__ w, const QuantJob quant) {
+  const unsigned route_blocks = gridDim.x - quant.blocks;
+  if (blockIdx.x >= route_blocks) {   // the blocks behind the routing blocks quantise the activations (QuantJob)
+    moe_quant_act_block(quant, blockIdx.x - route_blocks);
+    return;
+  }
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (t >= M) return;
@@ -141,7 +147,12 @@ template <int VPL>
 __global__ __launch_bounds__(kWavesPerBlock* MOE_WAVE) void route_sigmoid_grouped_kernel(
     const LogitSource src, const float* __restrict__ bias, int M, int E, int n_group,
     int topk_group, int k, int renorm, float routed_scale, int32_t* __restrict__ idx,
-    float* __restrict__ w) {
+    float* __restrict__ w, const QuantJob quant) {
+  const unsigned route_blocks = gridDim.x - quant.blocks;
+  if (blockIdx.x >= route_blocks) {   // the blocks behind the routing blocks quantise the activations (QuantJob)
+    moe_quant_act_block(quant, blockIdx.x - route_blocks);
+    return;
+  }
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   if (t >= M) return;
@@ -231,9 +242,10 @@ int check_route_args(const LogitSource& src, int M, int E, int k, const int32_t*
 
 }  // namespace
 
+static_assert(kWavesPerBlock * MOE_WAVE == 256, "a routing block doubles as a quantiser block of 256 pieces");
 #define DISPATCH_VPL(E, KERNEL, ...)                                                      \
   do {                                                                                    \
-    dim3 grid((M + kWavesPerBlock - 1) / kWavesPerBlock), block(kWavesPerBlock* MOE_WAVE); \
+    dim3 grid((M + kWavesPerBlock - 1) / kWavesPerBlock + qj.blocks), block(kWavesPerBlock* MOE_WAVE); \
     int vpl = ((E) + 63) / 64;                                                            \
     if (vpl <= 1) hipLaunchKernelGGL(KERNEL<1>, grid, block, 0, s, __VA_ARGS__);          \
     else if (vpl <= 2) hipLaunchKernelGGL(KERNEL<2>, grid, block, 0, s, __VA_ARGS__);     \
@@ -243,25 +255,28 @@ int check_route_args(const LogitSource& src, int M, int E, int k, const int32_t*
   } while (0)
 
 int moe_route_softmax_impl(const LogitSource& src, int M, int E, int k, int renorm, int32_t* idx, float* w,
-                           moe_stream_t stream) {
+                           moe_stream_t stream, const QuantJob* quant) {
   int rc = check_route_args(src, M, E, k, idx, w);
   if (rc) return rc;
+  MOE_REQUIRE(!quant || M > 0, MOE_ERR_BAD_SHAPE, "route: nothing to carry a quantisation with");
   if (M == 0) return MOE_OK;
   hipStream_t s = (hipStream_t)stream;
-  DISPATCH_VPL(E, route_softmax_kernel, src, M, E, k, renorm, idx, w);
+  const QuantJob qj = quant ? *quant : QuantJob{};
+  DISPATCH_VPL(E, route_softmax_kernel, src, M, E, k, renorm, idx, w, qj);
   return moe_check_hip(hipGetLastError(), "route_softmax launch");
 }
 
 extern "C" int moe_route_softmax_topk(const float* logits, int M, int E, int k, int renorm,
                                       int32_t* idx, float* w, moe_stream_t stream) {
-  return moe_route_softmax_impl(LogitSource{logits, nullptr, 0, E, nullptr, nullptr}, M, E, k, renorm, idx, w, stream);
+  return moe_route_softmax_impl(LogitSource{logits, nullptr, 0, E, nullptr, nullptr}, M, E, k, renorm, idx, w, stream, nullptr);
 }
 
 int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, int M, int E, int n_group,
                                    int topk_group, int k, int renorm, float routed_scale, int32_t* idx, float* w,
-                                   moe_stream_t stream) {
+                                   moe_stream_t stream, const QuantJob* quant) {
   int rc = check_route_args(src, M, E, k, idx, w);
   if (rc) return rc;
+  MOE_REQUIRE(!quant || M > 0, MOE_ERR_BAD_SHAPE, "route: nothing to carry a quantisation with");
   MOE_REQUIRE(n_group >= 1 && n_group <= 64 && E % n_group == 0, MOE_ERR_BAD_SHAPE,
               "route: n_group=%d must divide E=%d and be <= 64", n_group, E);
   MOE_REQUIRE(topk_group >= 1 && topk_group <= n_group, MOE_ERR_BAD_SHAPE,
@@ -270,8 +285,9 @@ int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, in
               "route: k=%d exceeds the %d experts of the kept groups", k, topk_group * (E / n_group));
   if (M == 0) return MOE_OK;
   hipStream_t s = (hipStream_t)stream;
+  const QuantJob qj = quant ? *quant : QuantJob{};
   DISPATCH_VPL(E, route_sigmoid_grouped_kernel, src, bias, M, E, n_group, topk_group, k, renorm,
-               routed_scale, idx, w);
+               routed_scale, idx, w, qj);
   return moe_check_hip(hipGetLastError(), "route_sigmoid_grouped launch");
 }
 
@@ -280,5 +296,5 @@ extern "C" int moe_route_sigmoid_grouped(const float* logits, const float* bias,
                                          float routed_scale, int32_t* idx, float* w,
                                          moe_stream_t stream) {
   return moe_route_sigmoid_grouped_impl(LogitSource{logits, nullptr, 0, E, nullptr, nullptr}, bias, M, E, n_group,
-                                        topk_group, k, renorm, routed_scale, idx, w, stream);
+                                        topk_group, k, renorm, routed_scale, idx, w, stream, nullptr);
 }
