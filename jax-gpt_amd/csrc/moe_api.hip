@@ -29,13 +29,6 @@ extern "C" const char* moe_last_error(void) { return g_err; }
 
 namespace {
 
-__global__ void dense_offsets_kernel(int32_t* off, int M) {
-  if (threadIdx.x == 0) {
-    off[0] = 0;
-    off[1] = M;
-  }
-}
-
 // One side stream per device, default priority, created on first use and kept for the life of the process.
 int side_stream(hipStream_t* out) {
   static std::mutex mu;
@@ -81,7 +74,7 @@ ForwardBuffers carve(void* ws, int M, int D, int E, int k, int I, int SI, bool r
   b.group_offsets = (int32_t*)c.take((size_t)(E + 1) * 4);
   b.sorted_token_ids = (int32_t*)c.take(R * 4);
   b.inv_perm = (int32_t*)c.take(R * 4);
-  b.dense_off = (int32_t*)c.take(8);
+  b.dense_off = (int32_t*)c.take(8);   // (stands in for the shared expert's group offsets, which its pre-built tile list makes unread)
   b.permute_ws_bytes = moe_permute_workspace_bytes(M, k, E);
   b.permute_ws = c.take(b.permute_ws_bytes);
   b.gemm_ws_bytes = moe_gemm_workspace_bytes((int)R, E, I > D ? I : D);
@@ -191,9 +184,8 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   // the shared expert's one group and its tile list (they depend on M alone: enqueued ahead of the quantiser where
   // the side stream runs it, so that nothing stands between the quantiser and the shared gate/up GEMM)
   auto list_shared = [&]() {
-    hipLaunchKernelGGL(dense_offsets_kernel, dim3(1), dim3(64), 0, side, b.dense_off, a->M);
     if (!rc_shared)
-      rc_shared = moe_gemm_build_tile_list(b.dense_off, 1, a->M, b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
+      rc_shared = moe_gemm_build_dense_tile_list(a->M, b.gemm_ws_shared, b.gemm_ws_shared_bytes, (moe_stream_t)side);
   };
   auto launch_shared = [&]() {
     GemmScales sc = moe_row_major_scales(a->D, a->SI);

@@ -236,7 +236,7 @@ int moe_route_sigmoid_grouped_impl(const LogitSource& src, const float* bias, in
 // own.  moe_gemm_tile_list describes the list the GEMMs of (R rows, E experts) expect in ws, so that the permutation
 // kernels, which hold every expert's row range anyway, can write it (moe_permute_impl) and no launch is spent on it.
 int moe_gemm_tile_list(int R, int E, void* ws, size_t ws_bytes, TileList* list);
-int moe_gemm_build_tile_list(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream);
+int moe_gemm_build_dense_tile_list(int R, void* ws, size_t ws_bytes, moe_stream_t stream);
 // the activation quantisers with an optional second copy of the scales, block-major in row order ((K/128, R): what
 // GemmScales{1, R} reads) -- spares the shared expert of a large batch the separate transposition
 int moe_quant_act_impl(const void* x_bf16, int R, int K, uint8_t* xq, float* sx, float* sx_blocked, moe_stream_t stream);

@@ -75,13 +75,16 @@ constexpr int ROTC = 2;       // MFMA groups by which wave set 1 trails wave set
 
 // One workgroup lists the row tiles of every expert (an expert's tiles side by side; which expert where: see
 // moe_tile_first); thread e owns expert e.
+// (dense_rows >= 0: one group of that many rows, whatever group_offsets holds -- the shared expert)
 __global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __restrict__ group_offsets, int E,
-                                                          TileList l) {
+                                                          TileList l, int dense_rows) {
   __shared__ int s_rows[1024];
   __shared__ int s_key[1024];
   const int e = threadIdx.x;
   int start = 0, rows = 0;
-  if (e < E) {
+  if (dense_rows >= 0) {
+    rows = e == 0 ? dense_rows : 0;
+  } else if (e < E) {
     start = group_offsets[e];
     rows = group_offsets[e + 1] - start;
   }
@@ -591,7 +594,7 @@ int launch(const uint8_t* xq, const float* sx, const int32_t* row_ids, const uin
               "gemm: one expert matrix and the activation array must each stay within 4 GB (N=%d K=%d R=%d)", N, K, R);
   if (R == 0) return MOE_OK;
   const TileList l = tile_list(ws, R, E);
-  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, l);
+  if (!list_built) hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, s, group_offsets, E, l, -1);
   static std::atomic<unsigned long long> lds_raised{0};
   if (int rc = moe_raise_lds_limit((const void*)grouped_gemm_kernel<MODE>, CLS_LDS_BYTES, lds_raised)) return rc;
   // An output that the memory-side cache (256 MB) cannot hold until the combine reads it goes past the caches
@@ -729,12 +732,12 @@ extern "C" int moe_gemm_down_fp8_layout(const uint8_t* hq, const float* sh, cons
   return moe_gemm_down_impl(hq, sh, w_down, sw_down, group_offsets, E, R, I, D, y_bf16, ws, ws_bytes, false, sc, stream);
 }
 
-// Builds, ahead of the GEMM launches, the list that they read from ws when they are told list_built = true.
-int moe_gemm_build_tile_list(const int32_t* group_offsets, int E, int R, void* ws, size_t ws_bytes, moe_stream_t stream) {
+// Builds, ahead of the GEMM launches, the list that they read from ws when they are told list_built = true:
+// one group of R rows (the shared expert).
+int moe_gemm_build_dense_tile_list(int R, void* ws, size_t ws_bytes, moe_stream_t stream) {
   TileList l;
-  if (int rc = moe_gemm_tile_list(R, E, ws, ws_bytes, &l)) return rc;
-  MOE_REQUIRE(group_offsets, MOE_ERR_NULL, "gemm tiles: null group offsets");
-  hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, group_offsets, E, l);
+  if (int rc = moe_gemm_tile_list(R, 1, ws, ws_bytes, &l)) return rc;
+  hipLaunchKernelGGL(build_tiles_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, (const int32_t*)nullptr, 1, l, R);
   return moe_check_hip(hipGetLastError(), "gemm tiles launch");
 }
 
