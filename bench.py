@@ -27,20 +27,37 @@ PEAK_FP8_TFLOPS = 5000.0     # MI355X dense fp8 MFMA (published)
 PEAK_HBM_GBS = 8000.0        # MI355X HBM3E (published)
 
 
-def measured_traffic(workload):
-    """HBM-side bytes per launch of the workload's dominant kernel (the routed gate/up grouped GEMM), as measured
-    with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: read at run time from the committed summary under profiles/,
-    which carries the commands and the calibration next to a line
-        traffic: workload=<name> kernel=gateup_routed fetch_bytes=<n> write_bytes=<n>
+def measured_traffic(workload, kernel="gateup_routed"):
+    """HBM-side bytes per launch of one of the workload's routed grouped GEMM launches (kernel = gateup_routed or
+    down_routed), as measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: read at run time from the committed
+    summary under profiles/, which carries the commands and the calibration next to a line
+        traffic: workload=<name> kernel=<kernel> fetch_bytes=<n> write_bytes=<n>
     Returns (bytes or None, the file it came from or None)."""
     import glob
     import re
     for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic*.txt"))):
         for ln in open(path):
-            m = re.match(r"\s*traffic:\s+workload=(\S+)\s+kernel=gateup_routed\s+fetch_bytes=(\d+)\s+write_bytes=(\d+)", ln)
-            if m and m.group(1) == workload:
-                return float(m.group(2)) + float(m.group(3)), os.path.relpath(path, ROOT)
+            m = re.match(r"\s*traffic:\s+workload=(\S+)\s+kernel=(\S+)\s+fetch_bytes=(\d+)\s+write_bytes=(\d+)", ln)
+            if m and m.group(1) == workload and m.group(2) == kernel:
+                return float(m.group(3)) + float(m.group(4)), os.path.relpath(path, ROOT)
     return None, None
+
+
+GATEUP_NAME = "grouped_gemm_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)"
+DOWN_NAME = "grouped_gemm_kernel<1>, routed launch (down, bf16 rows)"
+
+
+def kernel_roofline(bound, kern, workload, kernel_key, name):
+    """The roofline object of one launch timed alone (HIP events on the stream it is launched on): achieved =
+    algorithmic FLOPs (or algorithmic weight bytes) per launch / average launch duration."""
+    traffic, src = measured_traffic(workload, kernel_key)
+    if bound == "mfma":
+        ach, peak, unit = kern["tflops"], PEAK_FP8_TFLOPS, "TFLOP/s"
+    else:
+        ach, peak, unit = kern["gbs"], PEAK_HBM_GBS, "GB/s"
+    return {"bound": bound, "achieved": ach, "peak": peak, "unit": unit, "frac": ach / peak, "traffic": traffic,
+            "traffic_source": src, "kernel": name, "avg_launch_ms": kern["avg_launch_ms"],
+            "flops_per_launch": kern["flops_per_launch"], "algorithmic_bytes_per_launch": kern["bytes_per_launch"]}
 
 
 WORKLOADS = {
@@ -110,7 +127,7 @@ def timed(torch, fn, steps, warmup):
     return start.elapsed_time(stop) / steps, wall
 
 
-def run_workload(jg, torch, name, cfg, layer, steps, warmup):
+def run_workload(jg, torch, name, cfg, layer, steps, warmup, graph=True):
     experts, shared, bias, gen = layer
     x, logits = make_inputs(torch, cfg, gen)
     kw = dict(top_k=cfg["k"], experts=experts, shared=shared, routing=cfg["routing"], bias=bias,
@@ -136,6 +153,8 @@ def run_workload(jg, torch, name, cfg, layer, steps, warmup):
     # decode-sized batches, where a dozen dependent launches share a millisecond
     res["graph_ms_per_step"] = None
     try:
+        if not graph:
+            raise RuntimeError("not asked for")
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -177,6 +196,15 @@ def run_workload(jg, torch, name, cfg, layer, steps, warmup):
     k_bytes = touched * per_expert_bytes * 2 / 3
     res["gateup_kernel"] = dict(avg_launch_ms=k_ms, flops_per_launch=k_flops, tflops=k_flops / k_ms / 1e9,
                                 bytes_per_launch=k_bytes, gbs=k_bytes / k_ms / 1e6)
+    # the routed down launch, timed alone the same way, on the h that the gate/up launch wrote
+    hq, sh = jg.gemm_gateup_swiglu(xq, sxk, experts["gate_proj"], experts["up_proj"], sg["group_offsets"],
+                                   row_ids=sg["sorted_token_ids"], block_major=blocked)
+    d_ms, _ = timed(torch, lambda: jg.gemm_down(hq, sh, experts["down_proj"], sg["group_offsets"], block_major=blocked),
+                    steps, max(2, warmup // 2))
+    d_flops = 2.0 * R * D * I
+    d_bytes = touched * per_expert_bytes / 3
+    res["down_kernel"] = dict(avg_launch_ms=d_ms, flops_per_launch=d_flops, tflops=d_flops / d_ms / 1e9,
+                              bytes_per_launch=d_bytes, gbs=d_bytes / d_ms / 1e6)
     return res
 
 
@@ -216,17 +244,22 @@ def run_ep_shard(jg, torch, steps, warmup, seed=5):
     sxb = jg.gather_scales(sx)
     k_ms, _ = timed(torch, lambda: jg.gemm_gateup_swiglu(xq, sxb, experts["gate_proj"], experts["up_proj"], off,
                                                          block_major=True), steps, max(2, warmup // 2))
+    hq, sh = jg.gemm_gateup_swiglu(xq, sxb, experts["gate_proj"], experts["up_proj"], off, block_major=True)
+    d_ms, _ = timed(torch, lambda: jg.gemm_down(hq, sh, experts["down_proj"], off, block_major=True), steps, max(2, warmup // 2))
     flops = 6.0 * R * D * I
-    k_flops = 4.0 * R * D * I
+    k_flops, d_flops = 4.0 * R * D * I, 2.0 * R * D * I
     touched = int((group_sizes > 0).sum())
+    per_expert_bytes = 3 * D * I + 3 * (D // 128) * (I // 128) * 4
+    gk = dict(avg_launch_ms=k_ms, flops_per_launch=k_flops, tflops=k_flops / k_ms / 1e9,
+              bytes_per_launch=touched * per_expert_bytes * 2 / 3, gbs=touched * per_expert_bytes * 2 / 3 / k_ms / 1e6)
+    dk = dict(avg_launch_ms=d_ms, flops_per_launch=d_flops, tflops=d_flops / d_ms / 1e9,
+              bytes_per_launch=touched * per_expert_bytes / 3, gbs=touched * per_expert_bytes / 3 / d_ms / 1e6)
     return {"metric": "expert-parallel shard fp8 TFLOP/s (pre-dispatched rows, gate/up + down + combine)",
             "value": flops / ms / 1e9, "unit": "TFLOP/s", "ms_per_step": ms, "frac_of_peak": flops / ms / 1e9 / PEAK_FP8_TFLOPS,
             "config": {"workload": "ep_shard_skewed", "local_experts": E, "rows": R, "D": D, "I": I, "k": k, "tokens": M,
                        "touched_experts": touched, "largest_group": int(group_sizes.max()), "group_sizes": "Zipf(1.2)"},
-            "roofline": {"bound": "mfma", "achieved": k_flops / k_ms / 1e9, "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                         "frac": k_flops / k_ms / 1e9 / PEAK_FP8_TFLOPS, "traffic": None,
-                         "kernel": "grouped_gemm_kernel<0> (gate/up + SwiGLU + h quantisation), rows in expert order",
-                         "avg_launch_ms": k_ms, "flops_per_launch": k_flops}}
+            "roofline": kernel_roofline("mfma", gk, "ep_shard_skewed", "gateup_routed", GATEUP_NAME + ", rows in expert order"),
+            "down_kernel": kernel_roofline("mfma", dk, "ep_shard_skewed", "down_routed", DOWN_NAME)}
 
 
 def cpu_baseline(cfg, seconds_budget=25.0):
@@ -287,6 +320,15 @@ def main():
         dcfg = WORKLOADS["deepseek_v3_decode"]
         decode = run_workload(jg, torch, "deepseek_v3_decode", dcfg, layer, max(args.steps, 20), args.warmup)
         log(json.dumps(decode))
+    # the same two shapes under balanced routing (selection bias 0: every expert gets 256 +- 16 rows at prefill, about
+    # 221 experts of two or three rows are touched at decode), in the default run only
+    balanced = None
+    if args.workload == "deepseek_v3_prefill" and not args.no_extra and not args.no_decode and args.bias_std != 0.0:
+        flat = (layer[0], layer[1], torch.zeros_like(layer[2]), layer[3])
+        balanced = (run_workload(jg, torch, "deepseek_v3_prefill_balanced", cfg, flat, args.steps, args.warmup, graph=False),
+                    run_workload(jg, torch, "deepseek_v3_decode_balanced", WORKLOADS["deepseek_v3_decode"], flat,
+                                 max(args.steps, 20), args.warmup))
+        log(json.dumps(balanced))
     # the other two MFMA-bound configurations of the benchmark, measured in the same run (the default run only)
     qwen3 = ep_shard = None
     if args.workload == "deepseek_v3_prefill" and not args.no_extra:
@@ -298,20 +340,30 @@ def main():
         ep_shard = run_ep_shard(jg, torch, max(args.steps, 20), args.warmup)
         log(json.dumps(ep_shard))
 
-    gk = main_res["gateup_kernel"]
+    def prefill_obj(res, workload, cfg_):
+        return {"metric": "MoE layer fp8 TFLOP/s (prefill)", "value": res["tflops"], "unit": "TFLOP/s",
+                "ms_per_step": res["ms_per_step"], "graph_replay_ms_per_step": res["graph_ms_per_step"],
+                "frac_of_peak": res["tflops"] / PEAK_FP8_TFLOPS,
+                "config": {"workload": workload, **{k: cfg_[k] for k in ("M", "D", "E", "k", "I", "SI", "routing")},
+                           "touched_experts": res["touched_experts"]},
+                "roofline": kernel_roofline("mfma", res["gateup_kernel"], workload, "gateup_routed", GATEUP_NAME),
+                "down_kernel": kernel_roofline("mfma", res["down_kernel"], workload, "down_routed", DOWN_NAME)}
+
+    def decode_obj(res, workload):
+        return {"metric": "HBM GB/s over touched fp8 expert weights", "value": res["gbs"], "unit": "GB/s",
+                "ms_per_step": res["ms_per_step"], "graph_replay_ms_per_step": res["graph_ms_per_step"],
+                "graph_replay_value": res.get("graph_gbs"), "touched_experts": res["touched_experts"],
+                "weight_bytes": res["weight_bytes"], "frac_of_peak": res["gbs"] / PEAK_HBM_GBS,
+                "roofline": kernel_roofline("hbm", res["gateup_kernel"], workload, "gateup_routed", GATEUP_NAME),
+                "down_kernel": kernel_roofline("hbm", res["down_kernel"], workload, "down_routed", DOWN_NAME)}
+
+    tag = args.workload if args.bias_std == 0.1 else args.workload + "_bias%g" % args.bias_std
     if is_decode:
         metric, value, unit = "MoE layer HBM GB/s over touched fp8 expert weights (decode)", main_res["gbs"], "GB/s"
-        roof = {"bound": "hbm", "achieved": gk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": gk["gbs"] / PEAK_HBM_GBS, "traffic": None, "kernel": "gate/up grouped GEMM",
-                "avg_launch_ms": gk["avg_launch_ms"]}
+        head = decode_obj(main_res, tag)
     else:
         metric, value, unit = "MoE layer fp8 TFLOP/s (prefill)", main_res["tflops"], "TFLOP/s"
-        traffic, traffic_src = measured_traffic(args.workload) if args.bias_std == 0.1 else (None, None)
-        roof = {"bound": "mfma", "achieved": gk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                "frac": gk["tflops"] / PEAK_FP8_TFLOPS, "traffic": traffic, "traffic_source": traffic_src,
-                "kernel": "grouped_gemm_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
-                "algorithmic_bytes_per_launch": gk["bytes_per_launch"],
-                "avg_launch_ms": gk["avg_launch_ms"], "flops_per_launch": gk["flops_per_launch"]}
+        head = prefill_obj(main_res, tag, cfg)
     line = {
         "metric": metric, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": main_res["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -320,31 +372,17 @@ def main():
                    "touched_experts": main_res["touched_experts"], "bias_std": args.bias_std},
         "frac_of_peak": (value / PEAK_HBM_GBS) if is_decode else (value / PEAK_FP8_TFLOPS),
         "graph_replay_ms_per_step": main_res["graph_ms_per_step"],
-        "roofline": roof,
+        "roofline": head["roofline"], "down_kernel": head["down_kernel"],
     }
     if decode:
-        dk = decode["gateup_kernel"]
-        line["decode"] = {"metric": "HBM GB/s over touched fp8 expert weights", "value": decode["gbs"], "unit": "GB/s",
-                          "ms_per_step": decode["ms_per_step"], "graph_replay_ms_per_step": decode["graph_ms_per_step"],
-                          "graph_replay_value": decode.get("graph_gbs"), "touched_experts": decode["touched_experts"],
-                          "weight_bytes": decode["weight_bytes"], "frac_of_peak": decode["gbs"] / PEAK_HBM_GBS,
-                          "roofline": {"bound": "hbm", "achieved": dk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": dk["gbs"] / PEAK_HBM_GBS,
-                                       "traffic": measured_traffic("deepseek_v3_decode")[0],
-                                       "traffic_source": measured_traffic("deepseek_v3_decode")[1],
-                                       "algorithmic_bytes_per_launch": dk["bytes_per_launch"],
-                                       "kernel": "grouped_gemm_kernel<0>, routed launch (gate/up + SwiGLU + h quantisation)",
-                                       "avg_launch_ms": dk["avg_launch_ms"]}}
+        line["decode"] = decode_obj(decode, "deepseek_v3_decode")
     if qwen3:
-        qk = qwen3["gateup_kernel"]
-        line["qwen3_moe_prefill"] = {"metric": "MoE layer fp8 TFLOP/s (prefill)", "value": qwen3["tflops"], "unit": "TFLOP/s",
-                                     "ms_per_step": qwen3["ms_per_step"], "frac_of_peak": qwen3["tflops"] / PEAK_FP8_TFLOPS,
-                                     "config": {"workload": "qwen3_moe_prefill", **{k: WORKLOADS["qwen3_moe_prefill"][k] for k in ("M", "D", "E", "k", "I", "SI", "routing")},
-                                                "touched_experts": qwen3["touched_experts"]},
-                                     "roofline": {"bound": "mfma", "achieved": qk["tflops"], "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
-                                                  "frac": qk["tflops"] / PEAK_FP8_TFLOPS, "traffic": None,
-                                                  "kernel": "grouped_gemm_kernel<0>, routed launch", "avg_launch_ms": qk["avg_launch_ms"],
-                                                  "flops_per_launch": qk["flops_per_launch"]}}
+        line["qwen3_moe_prefill"] = prefill_obj(qwen3, "qwen3_moe_prefill", WORKLOADS["qwen3_moe_prefill"])
+    if balanced:
+        line["prefill_balanced"] = prefill_obj(balanced[0], "deepseek_v3_prefill_balanced", WORKLOADS["deepseek_v3_prefill"])
+        line["prefill_balanced"]["config"]["bias_std"] = 0.0
+        line["decode_balanced"] = decode_obj(balanced[1], "deepseek_v3_decode_balanced")
+        line["decode_balanced"]["bias_std"] = 0.0
     if ep_shard:
         line["ep_shard_skewed"] = ep_shard
     if not args.no_cpu:

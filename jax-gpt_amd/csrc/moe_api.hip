@@ -46,6 +46,35 @@ int side_stream(hipStream_t* out) {
   return MOE_OK;
 }
 
+// The events of a call with a shared expert (fork, activations quantised, join), kept per host thread and device
+// and created on first use: a call enqueues and returns on one thread, and a wait that is already enqueued keeps
+// the record it was enqueued after, so the thread's next call may record the same events again (calls of other
+// threads have their own).  They are never destroyed: the runtime may be gone by the time a thread ends.
+struct CallEvents {
+  hipEvent_t fork, quant, join;
+};
+int call_events(CallEvents** out) {
+  static thread_local CallEvents events[64] = {};
+  int dev = 0;
+  int rc = moe_check_hip(hipGetDevice(&dev), "forward: hipGetDevice");
+  if (rc) return rc;
+  if (dev < 0 || dev >= 64) return moe_set_error(MOE_ERR_HIP, "forward: device index %d out of range", dev);
+  CallEvents& ev = events[dev];
+  if (!ev.join) {
+    hipEvent_t made[3] = {};
+    for (int i = 0; i < 3; ++i) {
+      const hipError_t e = hipEventCreateWithFlags(&made[i], hipEventDisableTiming);
+      if (e != hipSuccess) {
+        for (int j = 0; j < i; ++j) (void)hipEventDestroy(made[j]);
+        return moe_check_hip(e, "forward: creating the fork/join events");
+      }
+    }
+    ev = CallEvents{made[0], made[1], made[2]};
+  }
+  *out = &ev;
+  return MOE_OK;
+}
+
 struct Carver {
   char* base;
   size_t used;
@@ -181,6 +210,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   hipEvent_t ev_fork = nullptr, ev_quant = nullptr, ev_join = nullptr;
   int rc_shared = MOE_OK;
   bool quant_joined = true;
+  bool side_forked = false;   // the side stream has been made to wait for work of this call on the caller's stream
   // the shared expert's one group and its tile list (they depend on M alone: enqueued ahead of the quantiser where
   // the side stream runs it, so that nothing stands between the quantiser and the shared gate/up GEMM)
   auto list_shared = [&]() {
@@ -215,24 +245,23 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     return rc;
   if (a->SI) {
     if ((rc = side_stream(&side))) return rc;
-    hipError_t e = hipEventCreateWithFlags(&ev_quant, hipEventDisableTiming);
-    if (e == hipSuccess) e = hipEventCreateWithFlags(&ev_join, hipEventDisableTiming);
-    if (e == hipSuccess && !small_batch) {
-      e = hipEventCreateWithFlags(&ev_fork, hipEventDisableTiming);
-      if (e == hipSuccess) e = hipEventRecord(ev_fork, main_s);
+    CallEvents* ev = nullptr;
+    if ((rc = call_events(&ev))) return rc;
+    ev_fork = ev->fork, ev_quant = ev->quant, ev_join = ev->join;
+    if (!small_batch) {
+      hipError_t e = hipEventRecord(ev_fork, main_s);
       if (e == hipSuccess) e = hipStreamWaitEvent(side, ev_fork, 0);
-      if (ev_fork) (void)hipEventDestroy(ev_fork);   // released once the recorded work has completed
-    }
-    if (e != hipSuccess) {
-      if (ev_quant) (void)hipEventDestroy(ev_quant);
-      if (ev_join) (void)hipEventDestroy(ev_join);
-      return moe_check_hip(e, "forward: fork");
+      if (e != hipSuccess) return moe_check_hip(e, "forward: fork");
+      side_forked = true;
     }
     if (small_batch) {
       if (!quant_in_route) {
         rc_shared = quantise(a, b, blocked_scales ? b.sx_blocked : nullptr, stream);
         if (!rc_shared) rc_shared = moe_check_hip(hipEventRecord(ev_quant, main_s), "forward: quant event");
-        if (!rc_shared) rc_shared = moe_check_hip(hipStreamWaitEvent(side, ev_quant, 0), "forward: fork");
+        if (!rc_shared) {
+          rc_shared = moe_check_hip(hipStreamWaitEvent(side, ev_quant, 0), "forward: fork");
+          side_forked = !rc_shared;
+        }
       }   // (else: the same record and wait follow the routing launch, below)
       shared_pending = true;
     } else {
@@ -245,18 +274,20 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
   } else if (!quant_in_route) {
     if ((rc = quantise(a, b, nullptr, stream))) return rc;
   }
-  // the join is enqueued on every path out of here, so that the caller's stream never loses track of the side stream
+  // Once the side stream has been forked off this call, the join is enqueued on every path out of here, so that the
+  // caller's stream (or the graph it is being captured into) never loses track of the side stream.  Before the
+  // fork the side stream holds nothing of this call, and a wait on it would tie the caller's stream -- under
+  // capture: the caller's graph -- to work that does not belong to it.
   auto join = [&](int code) {
     if (!a->SI) return code;
-    if (shared_pending && !code && !rc_shared) {
+    if (shared_pending && side_forked && !code && !rc_shared) {
       list_shared();
       launch_shared();
     }
     shared_pending = false;
+    if (!side_forked) return code ? code : rc_shared;
     hipError_t e1 = hipEventRecord(ev_join, side);
     hipError_t e2 = hipStreamWaitEvent(main_s, ev_join, 0);
-    (void)hipEventDestroy(ev_join);
-    (void)hipEventDestroy(ev_quant);
     if (code) return code;
     if (rc_shared) return rc_shared;
     if (e1 != hipSuccess) return moe_check_hip(e1, "forward: join");
@@ -294,6 +325,7 @@ extern "C" int moe_forward(const MoeForwardArgs* a, void* ws, size_t ws_bytes, m
     hipError_t e = hipEventRecord(ev_quant, main_s);
     if (e == hipSuccess) e = hipStreamWaitEvent(side, ev_quant, 0);
     if (e != hipSuccess) return join(moe_check_hip(e, "forward: quant event"));
+    side_forked = true;
   }
   // the permutation kernels also list the routed GEMMs' row tiles (they hold every expert's row range anyway)
   TileList tiles;

@@ -499,7 +499,7 @@ template <int MODE>
 __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const uint8_t* __restrict__ xq, const float* __restrict__ sx, const int32_t* __restrict__ row_ids,
     const uint8_t* __restrict__ w0, const float* __restrict__ sw0, const uint8_t* __restrict__ w1,
-    const float* __restrict__ sw1, const TileHeader* __restrict__ hdr, const TileEntry* __restrict__ tiles, int K,
+    const float* __restrict__ sw1, TileHeader* hdr, const TileEntry* __restrict__ tiles, int K,
     int N, void* __restrict__ out, float* __restrict__ out_scale, const GemmScales sc) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   // work items = (row tile, column block) pairs in [expert][column block][row tile] order, dealt to the 8 XCDs in
@@ -515,7 +515,7 @@ __global__ __launch_bounds__(NT, 1) void grouped_gemm_kernel(
     const int pool_items = (hdr->n_tiles - hdr->n_static) * ncb;
     if (pool_items == 0 || item_id - share_end >= moe_pool_workgroups(pool_items)) return;   // (uniform: the whole workgroup leaves)
     int* slot = (int*)lds;
-    if (threadIdx.x == 0) *slot = atomicAdd(const_cast<int*>(&hdr->pool_next[MODE]), 1);
+    if (threadIdx.x == 0) *slot = atomicAdd(&hdr->pool_next[MODE], 1);   // (the one field of the list a GEMM writes)
     __syncthreads();
     const int drawn = *slot;
     __syncthreads();   // (the work item's first copies overwrite the slot)

@@ -218,7 +218,7 @@ __global__ __launch_bounds__(kThreads) void permute_small_kernel(const int32_t* 
       if (i < wv) first += wave_tiles[i];
       all += wave_tiles[i];
     }
-    if (threadIdx.x == 0) {   // (32-row tiles: all alike; no pool)
+    if (threadIdx.x == 0) {   // (at most 2048 rows in all: the tiles are few and short, equal shares by count, no pool)
       const int n = all < tl.max_tiles ? all : tl.max_tiles;
       moe_tile_even_shares(tl.hdr, n, n);
     }

@@ -213,6 +213,8 @@ __global__ __launch_bounds__(256) void gather_scales_kernel(const float* __restr
 extern "C" int moe_gather_scales(const float* sx, const int32_t* row_ids, int n, int KB, float* out, moe_stream_t stream) {
   MOE_REQUIRE(n >= 0 && KB >= 1, MOE_ERR_BAD_SHAPE, "gather_scales: bad sizes n=%d KB=%d", n, KB);
   MOE_REQUIRE(n == 0 || (sx && out), MOE_ERR_NULL, "gather_scales: null pointer");
+  // (rows of a multiple of four scales are read 16 bytes at a time)
+  MOE_REQUIRE((KB & 3) || MOE_ALIGNED16(sx), MOE_ERR_BAD_ALIGN, "gather_scales: sx must be 16-byte aligned when KB is a multiple of 4");
   if (n == 0) return MOE_OK;
   hipLaunchKernelGGL(gather_scales_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, sx, row_ids,
                      n, KB, out);

@@ -113,6 +113,19 @@ def assert_h_close(hq, sh, ref_hq, ref_sh, what="h"):
     return frac
 
 
+# Intermediate sizes below this are outside the end-to-end contract: one e4m3 step on one element of h moves its
+# output row by up to ~0.45 / sqrt(I) of the row's size, so a single boundary case among a few hundred h elements
+# can exceed 1e-2 end to end (measured on random small layers: 2.3e-2 at I = 128, 1.5e-2 at I = 384, <= 7.5e-3 from
+# I = 512 up, which covers every configuration of the benchmark definition: I = 768, 1024, 2048).
+E2E_MIN_INTERMEDIATE = 512
+E2E_SMALL_TOL = 3e-2
+
+
+def end_to_end_tol(I, tol=1e-2):
+    """The bound on max|out - oracle| / max|oracle| of a whole-path call against the oracle on its own."""
+    return tol if I >= E2E_MIN_INTERMEDIATE else E2E_SMALL_TOL
+
+
 def check_layer_output(out, dbg, ref, rerun, tol=1e-2, shared_gate=None, residual=None):
     """End-to-end check of a whole-path call against the oracle.  The path rounds twice on the way (the SwiGLU
     output to fp8, the down GEMM's rows to bf16, as the reference's ragged_dot does), and a value that exact
@@ -127,7 +140,11 @@ def check_layer_output(out, dbg, ref, rerun, tol=1e-2, shared_gate=None, residua
           bit for bit (an f32 sum in slot order and one rounding);
       (4) the output against the oracle continued from the kernel's h: max-normalised error <= 1e-2, and the
           elementwise allclose wherever no bf16 step of a y row explains the difference (every exception is
-          counted; they stay below 0.1 % of the elements).
+          counted; they stay below 0.1 % of the elements);
+      (5) the output against the oracle ON ITS OWN (identical inputs, nothing taken from the kernel): max-normalised
+          error <= 1e-2, the tolerance of the benchmark definition, for intermediate sizes from
+          E2E_MIN_INTERMEDIATE up (end_to_end_tol; below that a single fp8 boundary case can exceed it and the
+          bound is E2E_SMALL_TOL).
     `ref` is the oracle on its own, `rerun(routed_h=, shared_h=)` the oracle continued from given intermediates.
     Returns (error of (4), end-to-end error against `ref`, fraction of h codes that differ)."""
     from oracle import moe_oracle as O_
@@ -152,7 +169,10 @@ def check_layer_output(out, dbg, ref, rerun, tol=1e-2, shared_gate=None, residua
     err = max_norm_err(got, ref2["out"])
     assert err <= tol, f"max-normalised error {err:.3e} > {tol:.3e}"
     assert_allclose_but_for_row_steps(got, ref2["out"], y, ref2["y"], ys, ref2["shared_out"], w, ref["inv_perm"], shared_gate, tol)
-    return err, max_norm_err(got, ref["out"]), frac
+    e2e = max_norm_err(got, ref["out"])
+    bound = end_to_end_tol(hq.shape[-1], tol)
+    assert e2e <= bound, f"end-to-end max-normalised error {e2e:.3e} > {bound:.1e} against the oracle on identical inputs"
+    return err, e2e, frac
 
 
 def _bf16_step(v):
@@ -176,7 +196,10 @@ def assert_allclose_but_for_row_steps(got, want, y, y_ref, ys, ys_ref, w, inv_pe
     rms = np.sqrt(np.mean(want ** 2))
     bound = tol * np.abs(want) + tol * rms
     diff = np.abs(got - want)
-    assert (diff <= bound + 1.01 * slack + _bf16_step(want)).all(), "an output element is outside the tolerance and no row step explains it"
+    # (where a y row differs, the rounded sum may also land one bf16 step of the output away: that step is granted
+    # only there)
+    widened = bound + np.where(slack > 0, 1.01 * slack + _bf16_step(want), 0.0)
+    assert (diff <= widened).all(), "an output element is outside the tolerance and no row step explains it"
     outside = diff > bound
     assert outside.mean() < 1e-3, f"{outside.mean():.3%} of the output elements lean on a row's rounding step"
     return int(outside.sum())

@@ -76,3 +76,58 @@ def test_static_scratch_rejects_what_does_not_fit(lib):
     rc = lib.moe_gemm_gateup_swiglu_fp8_static(one, one, None, one, one, one, one, one, 1024, 1 << 26, 128, 128, one, one, None)
     assert rc == -3, lib.moe_last_error().decode()
     assert "static scratch" in lib.moe_last_error().decode()
+
+
+def _static_call(lib, torch, bufs, hq, sh):
+    d_off, d_xq, d_sx, wg, sg, wu, su, E, R, D, I = bufs
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = lib.moe_gemm_gateup_swiglu_fp8_static(ptr(d_xq), ptr(d_sx), None, ptr(wg), ptr(sg), ptr(wu), ptr(su),
+                                               ptr(d_off), E, R, D, I, ptr(hq), ptr(sh), stream)
+    assert rc == 0, lib.moe_last_error().decode()
+
+
+def test_static_scratch_call_allocates_nothing_and_replays_from_a_graph(lib):
+    """What the entry point exists for: a call takes no device memory (free memory before = after, read from the
+    driver), and it can be captured in a HIP graph and replayed -- every replay, with eager calls in between, gives
+    the eager result bit for bit."""
+    import torch
+    torch.cuda.set_device(0)
+    off, xq, sx, ex = _case(4102, 5, 384, 256, [70, 0, 300, 1, 33])
+    E, I, D = ex["gate"][0].shape
+    R = int(off[-1])
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    bufs = (dev(off), dev(xq), dev(sx), dev(ex["gate"][0]), dev(ex["gate"][1]), dev(ex["up"][0]), dev(ex["up"][1]), E, R, D, I)
+    hq = torch.full((R, I), 0x7F, dtype=torch.uint8, device="cuda")
+    sh = torch.full((R, I // 128), -1.0, dtype=torch.float32, device="cuda")
+    _static_call(lib, torch, bufs, hq, sh)               # (first call on the device: looks up the array's address)
+    torch.cuda.synchronize()
+    eager = (hq.clone(), sh.clone())
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        _static_call(lib, torch, bufs, hq, sh)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"device memory changed across the calls: {free_before} -> {free_after}"
+    assert torch.equal(hq, eager[0]) and torch.equal(sh, eager[1])
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        _static_call(lib, torch, bufs, hq, sh)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _static_call(lib, torch, bufs, hq, sh)
+    for i in range(3):
+        print("   static replay", i, flush=True)
+        hq.fill_(0x7F)
+        sh.fill_(-1.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(hq, eager[0]) and torch.equal(sh, eager[1]), f"replay {i} differs from the eager call"
+        hq2, sh2 = torch.empty_like(hq), torch.empty_like(sh)     # eager work between the replays
+        _static_call(lib, torch, bufs, hq2, sh2)
+        torch.cuda.synchronize()
+        assert torch.equal(hq2, eager[0]) and torch.equal(sh2, eager[1])
