@@ -269,6 +269,41 @@ def run_ep_shard(jg, torch, steps, warmup, seed=5):
             "down_kernel": kernel_roofline("mfma", dk, "ep_shard_skewed", "down_routed", DOWN_NAME)}
 
 
+def run_probe(reps):
+    """`--probe`: the ceilings of the grouped GEMM's K loop on this box (jax-gpt_amd/csrc/moe_probe.hip: skeletons of
+    the loop on all 256 CUs, no epilogue, results meaningless).  Prints one JSON line with a list of measurements."""
+    import ctypes as C
+    path = os.path.join(ROOT, "jax-gpt_amd", "libmoe_probe.so")
+    if not os.path.exists(path):
+        import __graft_entry__
+        __graft_entry__.build()
+    lib = C.CDLL(path)
+    lib.moe_probe_variant_name.restype = C.c_char_p
+    lib.moe_probe_gemm_loop.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double),
+                                        C.POINTER(C.c_double)]
+    sources = ["every weight line an L2 hit", "weights from HBM, 4 workgroups share a slab", "weights from HBM, every workgroup its own slab"]
+    out = []
+    for random_data in (1, 0):
+        for v in range(lib.moe_probe_variants()):
+            name = lib.moe_probe_variant_name(v).decode()
+            for src in range(3):
+                if "compute only" in name and src:
+                    continue                      # (no copies: the source makes no difference)
+                if not random_data and not (name.startswith("A  structure") or "compute only" in name):
+                    continue                      # (constant data: only to show what the data cost)
+                ms, tf, gbs = C.c_double(), C.c_double(), C.c_double()
+                if lib.moe_probe_gemm_loop(v, src, random_data, reps, C.byref(ms), C.byref(tf), C.byref(gbs)):
+                    raise RuntimeError("moe_probe_gemm_loop failed")
+                rec = {"variant": name, "weights": sources[src] if "compute only" not in name else "-",
+                       "data": "random fp8 codes" if random_data else "constant bytes", "ms_per_launch": ms.value,
+                       "tflops": tf.value, "frac_of_fp8_peak": tf.value / PEAK_FP8_TFLOPS,
+                       "weight_tile_copy_gbs": gbs.value if "compute only" not in name else 0.0}
+                out.append(rec)
+                log(f"{rec['data']:17s} {rec['weights']:46s} {ms.value:7.3f} ms {tf.value:7.0f} TFLOP/s {rec['weight_tile_copy_gbs']:7.0f} GB/s  {name}")
+    print(json.dumps({"probe": "grouped GEMM K loop skeletons, 256 workgroups x 16 items x 56 K steps", "reps": reps,
+                      "peak_fp8_tflops": PEAK_FP8_TFLOPS, "measurements": out}), flush=True)
+
+
 def cpu_baseline(cfg, seconds_budget=25.0):
     """The reference's dataflow (oracle/reference_dataflow.py, a port) on the host cores, on a bounded
     sample of the prefill workload: a few experts at their mean row count."""
@@ -294,6 +329,12 @@ def main():
     ap.add_argument("--no-decode", action="store_true", help="skip the decode measurement")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the Qwen3-MoE prefill and the expert-parallel shard parts")
+    ap.add_argument("--parts", default="decode,balanced,qwen3,ep_shard",
+                    help="which measurements ride along with the default prefill workload (comma-separated subset of "
+                         "decode, balanced, qwen3, ep_shard; counter runs take one at a time so that a grid size names a launch)")
+    ap.add_argument("--probe", action="store_true",
+                    help="instead of the benchmark: time the skeletons of the grouped GEMM's K loop (compute pattern alone, "
+                         "copies from L2 / HBM, alternative structures) and print their rates as one JSON line")
     ap.add_argument("--bias-std", type=float, default=0.1,
                     help="standard deviation of the selection bias of sigmoid_grouped routing (0.1 = the workload as "
                          "specified: the same 7 of 8 groups win almost every token; 0 = balanced routing)")
@@ -303,6 +344,9 @@ def main():
               "GPU's shard); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    if args.probe:
+        run_probe(max(args.steps, 20) * 5)
+        return
     import torch
     import jax_gpt_amd as jg
     from jax_gpt_amd import _lib
@@ -323,14 +367,21 @@ def main():
     is_decode = args.workload.endswith("decode")
 
     decode = None
-    if not is_decode and not args.no_decode and args.workload == "deepseek_v3_prefill":
+    parts = set(p for p in args.parts.split(",") if p)
+    if args.no_decode:
+        parts -= {"decode", "balanced"}
+    if args.no_extra:
+        parts -= {"balanced", "qwen3", "ep_shard"}
+    if args.workload != "deepseek_v3_prefill":
+        parts = set()
+    if "decode" in parts:
         dcfg = WORKLOADS["deepseek_v3_decode"]
         decode = run_workload(jg, torch, "deepseek_v3_decode", dcfg, layer, max(args.steps, 20), args.warmup)
         log(json.dumps(decode))
     # the same two shapes under balanced routing (selection bias 0: every expert gets 256 +- 16 rows at prefill, about
     # 221 experts of two or three rows are touched at decode), in the default run only
     balanced = None
-    if args.workload == "deepseek_v3_prefill" and not args.no_extra and not args.no_decode and args.bias_std != 0.0:
+    if "balanced" in parts and args.bias_std != 0.0:
         flat = (layer[0], layer[1], torch.zeros_like(layer[2]), layer[3])
         balanced = (run_workload(jg, torch, "deepseek_v3_prefill_balanced", cfg, flat, args.steps, args.warmup, graph=False),
                     run_workload(jg, torch, "deepseek_v3_decode_balanced", WORKLOADS["deepseek_v3_decode"], flat,
@@ -338,12 +389,14 @@ def main():
         log(json.dumps(balanced))
     # the other two MFMA-bound configurations of the benchmark, measured in the same run (the default run only)
     qwen3 = ep_shard = None
-    if args.workload == "deepseek_v3_prefill" and not args.no_extra:
+    if parts & {"qwen3", "ep_shard"}:
         del layer
         torch.cuda.empty_cache()
+    if "qwen3" in parts:
         qcfg = WORKLOADS["qwen3_moe_prefill"]
         qwen3 = run_workload(jg, torch, "qwen3_moe_prefill", qcfg, make_layer(jg, torch, qcfg, seed=2), max(args.steps, 20), args.warmup)
         log(json.dumps(qwen3))
+    if "ep_shard" in parts:
         ep_shard = run_ep_shard(jg, torch, max(args.steps, 20), args.warmup)
         log(json.dumps(ep_shard))
 

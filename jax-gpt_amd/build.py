@@ -14,6 +14,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB_PATH = os.path.join(HERE, "libmoe_hip.so")
+# the timing probe of the grouped GEMM's K loop (`python bench.py --probe`): its own library, nothing of the product links it
+PROBE_PATH = os.path.join(HERE, "libmoe_probe.so")
 
 SOURCES = ["moe_api.hip", "moe_route.hip", "moe_router.hip", "moe_permute.hip", "moe_quant.hip", "moe_gemm.hip",
            "moe_combine.hip"]
@@ -52,10 +54,15 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
         if len(procs) >= jobs:
             _drain(procs)
     _drain(procs)
+    probe = [hipcc, *COMMON, *PER_FILE["moe_gemm.hip"], "-shared", os.path.join(CSRC, "moe_probe.hip"), "-o", PROBE_PATH]
+    if verbose:
+        print(" ".join(probe), flush=True)
+    procs.append(("moe_probe.hip", subprocess.Popen(probe, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
+    _drain(procs)
     return LIB_PATH
 
 
