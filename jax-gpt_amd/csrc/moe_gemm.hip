@@ -97,7 +97,7 @@ __global__ __launch_bounds__(1024) void build_tiles_kernel(const int32_t* __rest
 
 // ---- the kernel ------------------------------------------------------------------------------------------------
 //
-// LDS stage = [weight tile 256 x 128 B][activation tile 32 XF x 128 B][32 XF activation scales].
+// LDS = [ring of weight tiles 256 x 128 B][ring of (activation tile 32 XF x 128 B, its 32 XF activation scales)].
 // Tiles are row-major with 128-byte rows; the 16-byte chunk c of row r sits at chunk position
 // c ^ ((r >> 1) & 7).  A fragment lane (row fr = lane % 16, quarter fq = lane / 16) feeds the
 // MFMA with K bytes [16 fq, +16) and [64 + 16 fq, +16) of its row -- the same choice for both
@@ -126,20 +126,38 @@ __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chu
 // finished behind the next step's barrier, while that step's first fragments travel from LDS.
 template <int XF> struct Cls {
   static constexpr int BM = 32 * XF, HALF = BM / 2;
-  static constexpr int STAGE_X_OFF = W_TILE_BYTES;
-  static constexpr int STAGE_S_OFF = W_TILE_BYTES + BM * BK;
+  // Two rings: weight tiles (32 KB each) and activation tiles with their scales.  Where 160 KB allow it the weight
+  // ring is one stage deeper than the activation ring (160 to 224 rows: three weight stages, two activation
+  // stages): the weight tile is the one that may come from HBM, the activation tile is shared by the item's column
+  // blocks and comes from L2.  Measured on the loop's skeleton, weights two steps ahead instead of one: 5-7 % on a
+  // weight slab that four workgroups share or that a workgroup streams alone, nothing when every line is an L2 hit.
+  static constexpr int X_NST = XF >= 5 ? 2 : XF >= 2 ? 3 : 4;
+  static constexpr int W_NST = XF == 8 ? 2 : XF >= 2 ? 3 : 4;
+  static constexpr int X_PRE = X_NST - 1, W_PRE = W_NST - 1;   // steps that a copy runs ahead of its use
+  static constexpr int X_STAGE_S_OFF = BM * BK;                // the scales behind the tile
   // + 256: every copying wave copies 64 scale slots from its first one on (no lane mask, which would cut the
   // unrolled K step into blocks); the surplus lanes rewrite other waves' slots with the same values or land in this pad
-  static constexpr int STAGE_BYTES = STAGE_S_OFF + BM * 4 + 256;
-  static constexpr int NSTAGE = XF >= 5 ? 2 : XF >= 2 ? 3 : 4;
-  static constexpr int PRE = NSTAGE - 1;
+  static constexpr int X_STAGE_BYTES = BM * BK + BM * 4 + 256;
+  static constexpr int X_RING_OFF = W_NST * W_TILE_BYTES;
+  static constexpr int RING_BYTES = X_RING_OFF + X_NST * X_STAGE_BYTES;
   // Only wave set 0 (waves 0-3) issues copies: a copy instruction can hold its wave at the memory pipeline's door
   // while the L1's queue is full, and with one wave of each SIMD never there the matrix core always has a wave that
   // can feed it (2-3 % over all eight waves copying).  Wave v copies weight row groups [8v, 8v + 8), activation row
   // groups v, v + 4, ... and 64 scale slots.
   static constexpr int X_OPS = XF;                     // activation copies per copying wave and step
-  static constexpr int OPS = 8 + X_OPS + 1;            // + 8 weight row groups + 1 scale copy
-  static constexpr int RING_BYTES = NSTAGE * STAGE_BYTES;
+  static constexpr int XS_OPS = X_OPS + 1;             // + 1 scale copy
+  static constexpr int OPS = 8 + XS_OPS;               // + 8 weight row groups
+  // Copies complete in the order of their issue, so within a step those with the earlier deadline go first: with
+  // the deeper weight ring the activation copies (and scales), then the weights; with rings of one depth the
+  // weights first (they are the ones that may miss).
+  static constexpr bool X_FIRST = W_PRE > X_PRE;
+  static constexpr bool is_w(int i) { return X_FIRST ? i >= XS_OPS : i < 8; }
+  static constexpr int w_index(int i) { return X_FIRST ? i - XS_OPS : i; }
+  static constexpr bool is_s(int i) { return X_FIRST ? i == X_OPS : i == OPS - 1; }
+  static constexpr int x_index(int i) { return X_FIRST ? i : i - 8; }
+  // what may still be in flight when a step starts that found every later copy issued: the activation stages and
+  // weight stages of the steps after it
+  static constexpr int IN_FLIGHT = (X_PRE - 1) * XS_OPS + (W_PRE - 1) * 8;
   // copy operations issued after group g: spread over the first SPREAD groups of the step
   static constexpr int SPREAD = XF >= 6 ? XF / 2 : XF >= 3 ? 3 : XF;
   static constexpr int first(int g) { return g <= 0 ? 0 : g >= SPREAD ? OPS : (OPS * g) / SPREAD; }
@@ -148,7 +166,7 @@ constexpr int cmax(int a, int b) { return a > b ? a : b; }
 constexpr int CLS_RING = cmax(cmax(cmax(Cls<8>::RING_BYTES, Cls<7>::RING_BYTES), cmax(Cls<6>::RING_BYTES, Cls<5>::RING_BYTES)),
                               cmax(cmax(Cls<4>::RING_BYTES, Cls<3>::RING_BYTES), cmax(Cls<2>::RING_BYTES, Cls<1>::RING_BYTES)));
 constexpr int CLS_WSCALE_OFF = CLS_RING;                       // [2][MAX_KB] weight block scales of the work item
-constexpr int CLS_LDS_BYTES = CLS_RING + 2 * MAX_KB * 4;      // 151040; the epilogues stage through the ring (<= 128 KB)
+constexpr int CLS_LDS_BYTES = CLS_RING + 2 * MAX_KB * 4;      // 160000; the epilogues stage through the ring (<= 128 KB)
 static_assert(CLS_LDS_BYTES <= 160 * 1024, "LDS");
 
 struct Item { int expert, row_start, row_count, col_block; };
@@ -203,21 +221,33 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
     soff = (unsigned)g * (unsigned)sc.in_row * 4u;
   }
   const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);
+  // copies of step t's operands: weight row group w of this wave, activation row group x, the scales
+  auto copy_w = [&](int t, int w) {
+    dma16(wmat + (size_t)t * BK + (size_t)w * 8 * K, woff[w & 1], lds0 + (unsigned)(t % C::W_NST) * W_TILE_BYTES + (cv * 8 + w) * 1024u);
+  };
+  auto copy_x = [&](int t, int x) {
+    dma16(xq + (size_t)t * BK, xoff[x], lds0 + C::X_RING_OFF + (unsigned)(t % C::X_NST) * C::X_STAGE_BYTES + (x * 4 + cv) * 1024u);
+  };
+  auto copy_s = [&](int t) {
+    dma4((const uint8_t*)(sx + (size_t)t * sc.in_kb), soff,
+         lds0 + C::X_RING_OFF + (unsigned)(t % C::X_NST) * C::X_STAGE_BYTES + C::X_STAGE_S_OFF + sbase * 4u);
+  };
+  // operation i of the copies that step kb issues: each kind runs its ring's depth ahead of its use
   auto issue_op = [&](int kb, int i) {
-    const unsigned st = lds0 + (unsigned)(kb % C::NSTAGE) * C::STAGE_BYTES;
-    if (i < 8) dma16(wmat + (size_t)kb * BK + (size_t)i * 8 * K, woff[i & 1], st + (cv * 8 + i) * 1024u);
-    else if (i < 8 + C::X_OPS) {
-      const int grp = (i - 8) * 4 + cv;
-      dma16(xq + (size_t)kb * BK, xoff[i - 8], st + C::STAGE_X_OFF + grp * 1024u);
-    } else dma4((const uint8_t*)(sx + (size_t)kb * sc.in_kb), soff, st + C::STAGE_S_OFF + sbase * 4u);
+    if (C::is_w(i)) copy_w(kb + C::W_PRE, C::w_index(i));
+    else if (C::is_s(i)) copy_s(kb + C::X_PRE);
+    else copy_x(kb + C::X_PRE, C::x_index(i));
   };
   if (xj == 0) {
+    // what the steps before the first would have issued, in their order (completion is counted in issue order)
 #pragma unroll
-    for (int s = 0; s < C::PRE; ++s)
-      if (s < KB) {
+    for (int j = -C::W_PRE; j < 0; ++j) {
 #pragma unroll
-        for (int i = 0; i < C::OPS; ++i) issue_op(s, i);
+      for (int i = 0; i < C::OPS; ++i) {
+        const int t = j + (C::is_w(i) ? C::W_PRE : C::X_PRE);
+        if (t >= 0 && t < KB) issue_op(j, i);
       }
+    }
   }
 
   float* wscale = (float*)(lds + CLS_WSCALE_OFF);
@@ -272,18 +302,23 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
     constexpr int NH = ROT > 0 ? ROT : 1;
     v8i held[NH];
     float hc0[NH], hc1[NH];
+    // copy_c: what the step issues -- 2: every copy; 1: the activation tile and scales only (the deeper weight
+    // ring has reached the item's last K block); 0: nothing
     auto step = [&](int kb, auto first_c, auto copy_c) {
-      constexpr bool FIRST = decltype(first_c)::value, COPY = decltype(copy_c)::value && ISSUE;
-      constexpr bool TAIL = !decltype(copy_c)::value;
-      // stage kb has landed once only the copies of younger steps are outstanding
+      constexpr bool FIRST = decltype(first_c)::value;
+      constexpr int KIND = decltype(copy_c)::value;
+      constexpr bool COPY = KIND > 0 && ISSUE;
+      constexpr int NOPS = KIND == 2 ? C::OPS : C::XS_OPS;   // (KIND 1 exists only where the activation copies come first)
+      // stage kb of both rings has landed once only the copies of later steps are outstanding
       if (!ISSUE) {
         // (the copying waves wait for their copies before the barrier; this set has none in flight)
-      } else if (!TAIL || C::PRE == 1) {
-        wait_vm<(C::PRE - 1) * C::OPS>();   // (COPY steps: steps kb+1 .. kb+PRE-1 are in flight)
+      } else if (KIND == 2) {
+        wait_vm<C::IN_FLIGHT>();
       } else {
         const int rem = KB - 1 - kb;        // the last steps: fewer and fewer copies are in flight
-        if (C::PRE > 2 && rem >= 2) wait_vm<(C::PRE > 2 ? 2 : 0) * C::OPS>();
-        else if (rem >= 1) wait_vm<C::OPS>();
+        constexpr int one = (C::X_PRE > 1 ? C::XS_OPS : 0) + (C::W_PRE > 1 ? 8 : 0);   // the copies of one later step
+        if (rem >= 2) wait_vm<C::IN_FLIGHT>();
+        else if (rem == 1) wait_vm<one>();
         else wait_vm<0>();
       }
       if (ROT > 0) wait_lgkm0();      // this wave's reads of stage kb - 1 are done before anyone overwrites it
@@ -301,28 +336,31 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
             pc1 = hc1[i];
             if (COPY) {
 #pragma unroll
-              for (int o = C::first(i); o < C::first(i + 1); ++o) issue_op(kb + C::PRE, o);
+              for (int o = C::first(i); o < C::first(i + 1); ++o)
+                if (o < NOPS) issue_op(kb, o);
             }
             fence();
           }
         } else if (COPY) {
 #pragma unroll
-          for (int o = 0; o < C::first(ROT); ++o) issue_op(kb + C::PRE, o);
+          for (int o = 0; o < C::first(ROT); ++o)
+            if (o < NOPS) issue_op(kb, o);
         }
       }
-      const uint8_t* st = lds + (kb % C::NSTAGE) * C::STAGE_BYTES;
+      const uint8_t* wt = lds + (kb % C::W_NST) * W_TILE_BYTES;
+      const uint8_t* xs = lds + C::X_RING_OFF + (kb % C::X_NST) * C::X_STAGE_BYTES;
       const float s0 = ws0[kb], s1 = MODE == MODE_GATEUP ? ws1[kb] : s0;
-      const uint8_t* xt = st + C::STAGE_X_OFF + xj * 16 * BK;
+      const uint8_t* xt = xs + xj * 16 * BK;
       // Every wave of a wave set asks LDS for its first fragments at this moment: the reads come back in issue
       // order, so the first MFMA's operands (activation fragment 0, weight fragment 0) are asked for first and the
       // scales last; the FMAs that finish the previous step's last group run while the reads travel.
       v8i xf[2];
       xf[0] = read_frag(xt);
 #pragma unroll
-      for (int f = 0; f < 4; ++f) wf[f] = read_frag(st + wfrag_off[f]);
+      for (int f = 0; f < 4; ++f) wf[f] = read_frag(wt + wfrag_off[f]);
       float sxv[XF];
       {
-        const uint8_t* sp = st + C::STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4;
+        const uint8_t* sp = xs + C::X_STAGE_S_OFF + xj * HALF * 4 + fr * XF * 4;
         if constexpr (XF % 4 == 0) {
 #pragma unroll
           for (int j = 0; j < XF; j += 4) {
@@ -377,19 +415,37 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
         pc1 = sxv[j] * s1;
         if (COPY) {
 #pragma unroll
-          for (int o = C::first(ROT + j); o < C::first(ROT + j + 1); ++o) issue_op(kb + C::PRE, o);
+          for (int o = C::first(ROT + j); o < C::first(ROT + j + 1); ++o)
+            if (o < NOPS) issue_op(kb, o);
         }
         fence();
       }
     };
     constexpr std::true_type yes{};
     constexpr std::false_type no{};
-    const int n_copy = KB - C::PRE;   // steps 0 .. n_copy-1 issue copies
-    if (n_copy > 0) step(0, yes, yes);
-    else step(0, yes, no);
+    constexpr std::integral_constant<int, 2> all{};
+    constexpr std::integral_constant<int, 1> x_only{};
+    constexpr std::integral_constant<int, 0> none{};
+    const int n_all = KB - C::W_PRE;   // steps 0 .. n_all-1 issue every copy
+    const int n_x = KB - C::X_PRE;     // steps up to n_x-1 still issue the activation tile of a later step
+    if (n_all > 0) {
+      step(0, yes, all);
+    } else {
+      bool done = false;
+      if constexpr (C::X_FIRST) {
+        if (n_x > 0) {
+          step(0, yes, x_only);
+          done = true;
+        }
+      }
+      if (!done) step(0, yes, none);
+    }
     int kb = 1;
-    for (; kb < n_copy; ++kb) step(kb, no, yes);
-    for (; kb < KB; ++kb) step(kb, no, no);
+    for (; kb < n_all; ++kb) step(kb, no, all);
+    if constexpr (C::X_FIRST) {
+      for (; kb < n_x; ++kb) step(kb, no, x_only);
+    }
+    for (; kb < KB; ++kb) step(kb, no, none);
     if constexpr (ROT > 0) {   // the groups carried out of the last step
 #pragma unroll
       for (int i = 0; i < ROT; ++i) {
