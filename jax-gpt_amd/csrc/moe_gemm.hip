@@ -158,8 +158,11 @@ template <int XF> struct Cls {
   // what may still be in flight when a step starts that found every later copy issued: the activation stages and
   // weight stages of the steps after it
   static constexpr int IN_FLIGHT = (X_PRE - 1) * XS_OPS + (W_PRE - 1) * 8;
-  // copy operations issued after group g: spread over the first SPREAD groups of the step
-  static constexpr int SPREAD = XF >= 6 ? XF / 2 : XF >= 3 ? 3 : XF;
+  // copy operations issued after group g: spread over the first SPREAD groups of the step.  Rings of one depth must
+  // have the step's copies out early (they land before the next barrier or hold it up); with the deeper weight ring
+  // the weight copies have a step more, and an even spread over the whole step is best (all groups against the
+  // first three: gate/up -2 to -4 %, down -1 to -3 % on tiles of 160-224 rows; all at once: +2 %)
+  static constexpr int SPREAD = X_FIRST ? XF : XF >= 6 ? XF / 2 : XF >= 3 ? 3 : XF;
   static constexpr int first(int g) { return g <= 0 ? 0 : g >= SPREAD ? OPS : (OPS * g) / SPREAD; }
 };
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
