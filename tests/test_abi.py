@@ -131,3 +131,21 @@ def test_host_wrappers_refuse_cpu_tensors(dll):
         jg.route_softmax_topk(torch.zeros(4, 8), 2)
     with pytest.raises(RuntimeError, match="GPU"):
         jg.quant_act(torch.zeros(4, 128, dtype=torch.bfloat16))
+
+
+def test_probe_library_is_separate_and_loads(dll):
+    """The K-loop timing probe is a library of its own: it loads, exports its three entry points and nothing of
+    the product's, and the product library does not depend on it (no compute call is made here)."""
+    import subprocess
+    path = os.path.join(ROOT, "jax-gpt_amd", "libmoe_probe.so")
+    assert os.path.exists(path), "libmoe_probe.so is not built (python jax-gpt_amd/build.py)"
+    probe = C.CDLL(path)
+    probe.moe_probe_variant_name.restype = C.c_char_p
+    n = probe.moe_probe_variants()
+    assert n >= 5 and all(probe.moe_probe_variant_name(v) for v in range(n))
+    out = subprocess.run(["nm", "-D", "--defined-only", path], check=True, capture_output=True, text=True).stdout
+    exported = sorted(ln.split()[-1] for ln in out.splitlines() if ln.split()[-2:-1] == ["T"])
+    assert exported == ["moe_probe_gemm_loop", "moe_probe_variant_name", "moe_probe_variants"]
+    from jax_gpt_amd import _lib
+    needed = subprocess.run(["readelf", "-d", _lib.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    assert "moe_probe" not in needed
