@@ -96,8 +96,8 @@ __host__ __device__ inline void moe_tile_span(int rows, int nt, int t, int& star
 // as skewed as a biased router makes them, natural expert order leaves one XCD with up to a tenth more work than the
 // average, and the launch ends with its slowest XCD.  The experts are therefore ranked by size (ties: lower index
 // first) and dealt to eight bins in snake order (0..7, 7..0, ...); the list holds bin after bin.
-// Called by every thread of a workgroup with at least E threads; thread e owns expert e (rows = 0 for e >= E);
-// lds_rows and lds_key are int[blockDim.x] arrays in LDS.  Returns the index of expert e's first tile and, in
+// Called by every thread of a workgroup of 2^n >= E threads (at most 1024); thread e owns expert e (rows = 0 for
+// e >= E); lds_rows and lds_key are int[blockDim.x] arrays in LDS.  Returns the index of expert e's first tile and, in
 // *total_tiles, the length of the list, and writes the list header.
 //
 // The header's XCD shares are cut by cost, not by count: a row tile of u 32-row units costs about 8 + u (measured:
@@ -115,19 +115,43 @@ __device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int*
                                      TileHeader* hdr, int max_tiles) {
   __shared__ long long cut_q[9];
   __shared__ int tail_tiles[kTailRounds];   // tiles of the last, last but one, ... round of the ranking
+  __shared__ int sums[4];                   // non-empty experts; tiles, tiles outside the pool and their cost
+  __shared__ int acc_first[1024], acc_cost[1024];
+  // The two walks over all experts (the ranking; the tiles and cost in front of an expert) are shared out: with
+  // epad = E rounded up to a power of two (at least a wavefront), the workgroup's threads form blockDim / epad parts,
+  // thread (part, e2) walks the part's slice of the experts on behalf of expert e2, and the parts' sums meet in LDS
+  // (one thread per expert walking them all: 12 us of a 17 us launch for 128 experts).
+  int epad = 64;
+  while (epad < E) epad <<= 1;
+  const int parts = (int)blockDim.x / epad;          // >= 1: the caller has at least E threads, a power of two of them
+  const int e2 = e & (epad - 1), part = e / epad;
+  const int span = (epad + parts - 1) / parts;
+  const int o0 = part * span, o1 = o0 + span < E ? o0 + span : E;
+  const bool helper = part < parts && e2 < E;
   lds_rows[e] = e < E ? rows : 0;
+  lds_key[e] = 0;   // (first the ranks' accumulator)
+  acc_first[e] = 0;
+  acc_cost[e] = 0;
+  if (e < 4) sums[e] = 0;
   if (e < kTailRounds) tail_tiles[e] = 0;
   __syncthreads();
-  int key = e;
-  int rank = 0, nz = 0;
-  if (e < E) {
+  if (helper) {
+    const int mine = lds_rows[e2];
+    int ahead = 0;
 #pragma unroll 8
-    for (int o = 0; o < E; ++o) {
+    for (int o = o0; o < o1; ++o) {
       const int r = lds_rows[o];
-      rank += (r > rows || (r == rows && o < e)) ? 1 : 0;
-      nz += r > 0 ? 1 : 0;
+      ahead += (r > mine || (r == mine && o < e2)) ? 1 : 0;
     }
+    if (ahead) atomicAdd(&lds_key[e2], ahead);
   }
+  {
+    const unsigned long long busy = __ballot(e < E && rows > 0);
+    if ((e & 63) == 0 && busy) atomicAdd(&sums[0], __popcll(busy));
+  }
+  __syncthreads();
+  int key = e;
+  const int rank = lds_key[e], nz = sums[0];
   const int nr = (nz + 7) >> 3;   // rounds that hold a non-empty expert
   const int tail = nr / 4 < kTailRounds ? nr / 4 : kTailRounds;   // (3 rounds = 24 experts over the 8 bins; 6 measured no better)
   const int round = rank >> 3;
@@ -155,24 +179,36 @@ __device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int*
     key = ((round & 1) ? 7 - posn : posn) * 128 + pos;   // E <= 1024: at most 128 rounds
   }
   lds_key[e] = key;
-  __syncthreads();
-  int first = 0, total = 0, n_static = 0;
-  int cost_before = 0, cost_all = 0;
-  if (e < E) {   // (the threads past the last expert only keep the barriers company)
-#pragma unroll 8
-    for (int o = 0; o < E; ++o) {
-      const int t = moe_tile_count(lds_rows[o]);
-      const bool fixed = lds_key[o] < 1024;   // (not in the pool)
-      const int c = fixed ? 8 * t + ((lds_rows[o] + 31) >> 5) : 0;
-      const bool before = lds_key[o] < key;
-      total += t;
-      n_static += fixed ? t : 0;
-      cost_all += c;
-      first += before ? t : 0;
-      cost_before += before ? c : 0;
+  if (e < E) {   // the whole list's tiles, and the tiles and cost of the fixed shares (outside the pool)
+    const int t = moe_tile_count(rows);
+    if (t) {
+      atomicAdd(&sums[1], t);
+      if (key < 1024) {
+        atomicAdd(&sums[2], t);
+        atomicAdd(&sums[3], moe_tile_cost(rows));
+      }
     }
   }
-  *total_tiles = total;   // (valid for e < E)
+  __syncthreads();
+  if (helper) {
+    const int key2 = lds_key[e2];
+    int tiles_before = 0, cost_before_part = 0;
+#pragma unroll 8
+    for (int o = o0; o < o1; ++o) {
+      const int ko = lds_key[o], ro = lds_rows[o];
+      const int t = moe_tile_count(ro);
+      const int c = ko < 1024 ? 8 * t + ((ro + 31) >> 5) : 0;   // (not in the pool)
+      const bool before = ko < key2;
+      tiles_before += before ? t : 0;
+      cost_before_part += before ? c : 0;
+    }
+    if (tiles_before) atomicAdd(&acc_first[e2], tiles_before);
+    if (cost_before_part) atomicAdd(&acc_cost[e2], cost_before_part);
+  }
+  __syncthreads();
+  const int first = acc_first[e], cost_before = acc_cost[e];
+  const int total = sums[1], n_static = sums[2], cost_all = sums[3];
+  *total_tiles = total;
   // cut k sits where the cost of the fixed shares reaches k/8 of their whole: inside exactly one expert, whose
   // thread places it
   if (e < E && rows > 0 && key < 1024) {

@@ -113,10 +113,10 @@ __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chu
 // One launch, row tiles of every height.  A work item's row tile (at most 256 rows, near-equal cuts of its
 // expert) is served by the smallest of eight compiled tile classes that holds it -- 32 XF rows, XF = 1 .. 8 MFMA
 // groups per wave and K step -- each a branch-free, fully unrolled K loop of its own with its own LDS ring: the
-// short classes have short activation tiles and use the room for more stages (160 rows and more: two stages,
-// copies one K step ahead; 64 to 128 rows: three stages, two steps ahead; 32 rows: four stages, three steps
-// ahead), because an item of a few rows only streams its 256 weight rows and lives on the bytes it keeps in
-// flight.  Rows past the end of a tile are multiplied like the others (their copies re-read the tile's last
+// short classes have short activation tiles and use the room for more stages (256 rows: two stages; 160 to 224
+// rows: three weight stages, two activation stages; 64 to 128 rows: three stages, copies two steps ahead; 32 rows:
+// four stages, three steps ahead), because an item of a few rows only streams its 256 weight rows and lives on the
+// bytes it keeps in flight.  Rows past the end of a tile are multiplied like the others (their copies re-read the tile's last
 // row) and never stored.
 //
 // K step of a wave: XF groups; group j = its four weight fragments against activation fragment j (4 MFMAs, results
@@ -124,7 +124,7 @@ __device__ __forceinline__ int swz(int row, int chunk) { return row * BK + ((chu
 // group j + 1 -- FMA quadruple f just before MFMA f, which overwrites p[f] -- so the matrix core works on the next
 // group while the vector ALU finishes the last one, with one set of result registers.  The last group of a step is
 // finished behind the next step's barrier, while that step's first fragments travel from LDS.
-template <int XF> struct Cls {
+template <int XF, int MODE = MODE_GATEUP> struct Cls {
   static constexpr int BM = 32 * XF, HALF = BM / 2;
   // Two rings: weight tiles (32 KB each) and activation tiles with their scales.  Where 160 KB allow it the weight
   // ring is one stage deeper than the activation ring (160 to 224 rows: three weight stages, two activation
@@ -133,7 +133,19 @@ template <int XF> struct Cls {
   // weight slab that four workgroups share or that a workgroup streams alone, nothing when every line is an L2 hit.
   static constexpr int X_NST = XF >= 5 ? 2 : XF >= 2 ? 3 : 4;
   static constexpr int W_NST = XF == 8 ? 2 : XF >= 2 ? 3 : 4;
-  static constexpr int X_PRE = X_NST - 1, W_PRE = W_NST - 1;   // steps that a copy runs ahead of its use
+  // A weight stage is read once per step: every wave loads its four weight fragments into registers when it enters
+  // the step, and from then on the stage is free.  With W_EARLY the next tenant's copies are issued right there, in
+  // the middle of the step, and not behind the next barrier: the weights of step kb + 2 are then in flight while step
+  // kb still computes, as if the ring were a stage deeper, in the same LDS.  The weight rows that wave (wi, 0) copies
+  // are read by itself and by wave (wi, 1) alone, so the release is a word in LDS between those two (early_flag)
+  // and no barrier.  Only the 256-row class of the gate/up GEMM, which has no room for a third stage: -4.5 % where
+  // every workgroup streams its own weight slab, -3 % where 8 row tiles share one, nothing on the mixed tile
+  // heights of skewed routing; the down GEMM (16 K steps at the DeepSeek-V3 shape) gained 2 % in the first case and
+  // lost 1 % in the second, and the classes with three weight stages cannot gain: their copies complete in issue
+  // order behind the activation copies of the step before, which must have landed a step earlier.
+  static constexpr bool W_EARLY = XF == 8 && MODE == MODE_GATEUP;
+  static constexpr int EARLY_G = 3;   // the group behind which the weight copies of a W_EARLY step begin (2 and 4: within 1 %)
+  static constexpr int X_PRE = X_NST - 1, W_PRE = W_NST - 1 + (W_EARLY ? 1 : 0);   // steps that a copy runs ahead of its use
   static constexpr int X_STAGE_S_OFF = BM * BK;                // the scales behind the tile
   // + 256: every copying wave copies 64 scale slots from its first one on (no lane mask, which would cut the
   // unrolled K step into blocks); the surplus lanes rewrite other waves' slots with the same values or land in this pad
@@ -142,8 +154,8 @@ template <int XF> struct Cls {
   static constexpr int RING_BYTES = X_RING_OFF + X_NST * X_STAGE_BYTES;
   // Only wave set 0 (waves 0-3) issues copies: a copy instruction can hold its wave at the memory pipeline's door
   // while the L1's queue is full, and with one wave of each SIMD never there the matrix core always has a wave that
-  // can feed it (2-3 % over all eight waves copying).  Wave v copies weight row groups [8v, 8v + 8), activation row
-  // groups v, v + 4, ... and 64 scale slots.
+  // can feed it (2-3 % over all eight waves copying).  Wave v copies 8 weight row groups (the rows that it reads
+  // itself), activation row groups v, v + 4, ... and 64 scale slots.
   static constexpr int X_OPS = XF;                     // activation copies per copying wave and step
   static constexpr int XS_OPS = X_OPS + 1;             // + 1 scale copy
   static constexpr int OPS = 8 + XS_OPS;               // + 8 weight row groups
@@ -163,13 +175,19 @@ template <int XF> struct Cls {
   // the weight copies have a step more, and an even spread over the whole step is best (all groups against the
   // first three: gate/up -2 to -4 %, down -1 to -3 % on tiles of 160-224 rows; all at once: +2 %)
   static constexpr int SPREAD = X_FIRST ? XF : XF >= 6 ? XF / 2 : XF >= 3 ? 3 : XF;
-  static constexpr int first(int g) { return g <= 0 ? 0 : g >= SPREAD ? OPS : (OPS * g) / SPREAD; }
+  // (W_EARLY: the activation copies and scales behind groups 0 .. EARLY_G - 1, the weight copies behind the rest)
+  static constexpr int first(int g) {
+    if (W_EARLY)
+      return g <= 0 ? 0 : g < EARLY_G ? (XS_OPS * g) / EARLY_G : g >= XF ? OPS : XS_OPS + (8 * (g - EARLY_G)) / (XF - EARLY_G);
+    return g <= 0 ? 0 : g >= SPREAD ? OPS : (OPS * g) / SPREAD;
+  }
 };
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 constexpr int CLS_RING = cmax(cmax(cmax(Cls<8>::RING_BYTES, Cls<7>::RING_BYTES), cmax(Cls<6>::RING_BYTES, Cls<5>::RING_BYTES)),
                               cmax(cmax(Cls<4>::RING_BYTES, Cls<3>::RING_BYTES), cmax(Cls<2>::RING_BYTES, Cls<1>::RING_BYTES)));
 constexpr int CLS_WSCALE_OFF = CLS_RING;                       // [2][MAX_KB] weight block scales of the work item
-constexpr int CLS_LDS_BYTES = CLS_RING + 2 * MAX_KB * 4;      // 160000; the epilogues stage through the ring (<= 128 KB)
+constexpr int CLS_FLAG_OFF = CLS_WSCALE_OFF + 2 * MAX_KB * 4;  // [4] early_flag: the step whose weight fragments wave (wi, 1) holds, + 1
+constexpr int CLS_LDS_BYTES = CLS_FLAG_OFF + 16;              // 160016; the epilogues stage through the ring (<= 128 KB)
 static_assert(CLS_LDS_BYTES <= 160 * 1024, "LDS");
 
 struct Item { int expert, row_start, row_count, col_block; };
@@ -180,7 +198,7 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
                                           const uint8_t* __restrict__ w0, const float* __restrict__ sw0,
                                           const uint8_t* __restrict__ w1, const float* __restrict__ sw1, int K, int N,
                                           void* __restrict__ out, float* __restrict__ out_scale, const GemmScales sc) {
-  using C = Cls<XF>;
+  using C = Cls<XF, MODE>;
   constexpr int BM = C::BM, HALF = C::HALF;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -190,14 +208,16 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   const int e = item.expert;
   const int wrow0 = MODE == MODE_GATEUP ? item.col_block * 128 : item.col_block * 256;
 
-  // ---- copy sources: copying wave cv (waves 0-3; 4-7 compute the same values and never use them) fills weight row
-  // groups [8 cv, 8 cv + 8), activation row groups cv, cv + 4, ... and 64 scale slots
+  // ---- copy sources: copying wave cv (waves 0-3; 4-7 compute the same values and never use them) fills the weight
+  // rows that the waves wi = cv read (down: tile rows [64 cv, +64); gate/up: [32 cv, +32) of the gate half and of
+  // the up half), activation row groups cv, cv + 4, ... and 64 scale slots
   const int drow = lane >> 3, dchunk = lane & 7;
   const int cv = wave & 3;
-  const uint8_t* wmat = (MODE == MODE_GATEUP && cv >= 2 ? w1 : w0) + (size_t)e * N * K;   // uniform
+  const uint8_t* wmat = w0 + (size_t)e * N * K;   // uniform
+  const uint8_t* wmat1 = MODE == MODE_GATEUP ? w1 + (size_t)e * N * K : wmat;
   unsigned woff[2];
   {
-    int grow = MODE == MODE_GATEUP ? wrow0 + ((cv * 64) & 127) : wrow0 + cv * 64;
+    int grow = MODE == MODE_GATEUP ? wrow0 + cv * 32 : wrow0 + cv * 64;
     if (MODE == MODE_DOWN && grow >= N) grow = N - 64;   // (a half-full last column block: re-read valid rows)
     const int piece = dchunk ^ (drow >> 1);
     woff[0] = (unsigned)(grow + drow) * (unsigned)K + piece * 16;
@@ -226,7 +246,11 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
   const unsigned lds0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)lds);
   // copies of step t's operands: weight row group w of this wave, activation row group x, the scales
   auto copy_w = [&](int t, int w) {
-    dma16(wmat + (size_t)t * BK + (size_t)w * 8 * K, woff[w & 1], lds0 + (unsigned)(t % C::W_NST) * W_TILE_BYTES + (cv * 8 + w) * 1024u);
+    if (MODE == MODE_GATEUP)   // row groups 0-3 of the wave's gate rows, then of its up rows (tile rows 128 ..)
+      dma16((w < 4 ? wmat : wmat1) + (size_t)t * BK + (size_t)(w & 3) * 8 * K, woff[w & 1],
+            lds0 + (unsigned)(t % C::W_NST) * W_TILE_BYTES + ((w < 4 ? 0 : 16) + cv * 4 + (w & 3)) * 1024u);
+    else
+      dma16(wmat + (size_t)t * BK + (size_t)w * 8 * K, woff[w & 1], lds0 + (unsigned)(t % C::W_NST) * W_TILE_BYTES + (cv * 8 + w) * 1024u);
   };
   auto copy_x = [&](int t, int x) {
     dma16(xq + (size_t)t * BK, xoff[x], lds0 + C::X_RING_OFF + (unsigned)(t % C::X_NST) * C::X_STAGE_BYTES + (x * 4 + cv) * 1024u);
@@ -253,6 +277,9 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
     }
   }
 
+  volatile int* early_flag = (volatile int*)(lds + CLS_FLAG_OFF);
+  if (C::W_EARLY && tid < 4) early_flag[tid] = 0;
+  const unsigned my_flag = lds0 + CLS_FLAG_OFF + wi * 4;
   float* wscale = (float*)(lds + CLS_WSCALE_OFF);
   for (int i = tid; i < 2 * KB; i += NT) {
     const int h = i >= KB, kk = h ? i - KB : i;
@@ -416,12 +443,28 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
         }
         pc0 = sxv[j] * s0;
         pc1 = sxv[j] * s1;
+        if (C::W_EARLY && COPY && KIND == 2 && ROT + j == C::EARLY_G) {
+          // The weight copies from here on overwrite the stage that this step reads: this wave is past its own
+          // fragment loads; the other reader of its rows, wave (wi, 1), says so through early_flag.  (It entered the
+          // step through the same barrier and signals without waiting for anyone: the loop ends.  Inline assembly
+          // so that the unrolled step stays one block for the scheduler.)
+          fence();
+          int seen;
+          asm volatile("1:\n\tds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)\n\tv_cmp_ge_i32 vcc, %2, %0\n\ts_cbranch_vccnz 1b"
+                       : "=&v"(seen) : "v"(my_flag), "s"(kb) : "vcc", "memory");
+          fence();
+        }
         if (COPY) {
 #pragma unroll
           for (int o = C::first(ROT + j); o < C::first(ROT + j + 1); ++o)
             if (o < NOPS) issue_op(kb, o);
         }
         fence();
+        if (C::W_EARLY && !ISSUE && j == 0) {
+          // behind the MFMAs of the first group with this step's weights: all four weight fragments are in registers
+          early_flag[wi] = kb + 1;   // (every lane, one value: no branch)
+          fence();
+        }
       }
     };
     constexpr std::true_type yes{};

@@ -56,18 +56,28 @@ __global__ __launch_bounds__(kThreads) void hist_kernel(const int32_t* __restric
   for (int e = threadIdx.x; e < E; e += kThreads) chunk_hist[(size_t)blockIdx.x * E + e] = hist[e];
 }
 
-// one workgroup: thread e owns expert e (loop if E > blockDim)
+// one workgroup: thread e owns expert e.  With `cached` the (chunks x E) counts travel through LDS (kScanCacheInts
+// says when they fit): every thread of the workgroup loads and stores a share of them, coalesced, in one round of
+// independent accesses, and the per-expert walks over the chunks run on LDS.  Otherwise thread e walks its column
+// in global memory, in batches of independent loads (one load at a time would pay a memory round trip per chunk).
+constexpr int kScanCacheInts = 8192;   // 32 KB of dynamic LDS beside the static arrays (this kernel's and the tile helper's)
 __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk_hist, int n_chunks, int E,
                                                     int32_t* __restrict__ group_sizes,
-                                                    int32_t* __restrict__ group_offsets, TileList tl) {
+                                                    int32_t* __restrict__ group_offsets, TileList tl, int cached) {
+  extern __shared__ int cache[];   // [n_chunks][E] when cached
   __shared__ int tot[kMaxE];
   __shared__ int wave_tot[kMaxE / MOE_WAVE];
   __shared__ int tile_key[kMaxE];
   const int e = threadIdx.x;
-  // (the chunk loops read in batches of independent loads: one load at a time would pay a memory round trip per chunk)
   constexpr int kBatch = 8;
+  const int n_counts = n_chunks * E;
   int total = 0;
-  if (e < E) {
+  if (cached) {
+    for (int i = threadIdx.x; i < n_counts; i += kMaxE) cache[i] = chunk_hist[i];
+    __syncthreads();
+    if (e < E)
+      for (int c = 0; c < n_chunks; ++c) total += cache[c * E + e];
+  } else if (e < E) {
     for (int c0 = 0; c0 < n_chunks; c0 += kBatch) {
       int v[kBatch];
 #pragma unroll
@@ -75,8 +85,8 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
 #pragma unroll
       for (int i = 0; i < kBatch; ++i) total += v[i];
     }
-    group_sizes[e] = total;
   }
+  if (e < E) group_sizes[e] = total;
   // exclusive scan of totals over experts: wave scan + scan of wave totals
   const int lane = e & 63, wv = e >> 6;
   int incl = e < E ? total : 0;
@@ -94,7 +104,21 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
   if (e < E) {
     group_offsets[e] = excl;
     if (e == E - 1) group_offsets[E] = excl + total;
-    int run = excl;   // counts -> absolute first position of the expert's rows within each chunk, in place
+  }
+  // counts -> absolute first position of the expert's rows within each chunk, in place
+  if (cached) {
+    if (e < E) {
+      int run = excl;
+      for (int c = 0; c < n_chunks; ++c) {
+        const int v = cache[c * E + e];
+        cache[c * E + e] = run;
+        run += v;
+      }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < n_counts; i += kMaxE) chunk_hist[i] = cache[i];
+  } else if (e < E) {
+    int run = excl;
     for (int c0 = 0; c0 < n_chunks; c0 += kBatch) {
       int v[kBatch];
 #pragma unroll
@@ -117,36 +141,53 @@ __global__ __launch_bounds__(kMaxE) void scan_kernel(int32_t* __restrict__ chunk
   }
 }
 
+// Each wave places a contiguous quarter of the chunk, in flat order, from counters of its own: the waves first count
+// their quarters, a prefix over the waves turns the counts into each wave's first position per expert, and from there
+// on no wave waits for another (taking turns round by round cost two workgroup barriers per wave and round).
+constexpr int kWaveSpan = kChunk / kWaves;        // flat entries per wave
+constexpr int kWaveRounds = kWaveSpan / MOE_WAVE;
 __global__ __launch_bounds__(kThreads) void scatter_kernel(const int32_t* __restrict__ ids, int R, int E, int k,
                                                           const int32_t* __restrict__ chunk_base,
                                                           int32_t* __restrict__ sorted_token_ids,
                                                           int32_t* __restrict__ sort_order,
                                                           int32_t* __restrict__ inv_perm) {
-  extern __shared__ int smem[];  // next[E]: next free output position per expert within this chunk
-  int* next = smem;
-  for (int e = threadIdx.x; e < E; e += kThreads) next[e] = chunk_base[(size_t)blockIdx.x * E + e];
-  __syncthreads();
+  extern __shared__ int smem[];  // [kWaves][E]: a wave's counts, then its next free output position per expert
   const int bits = ilog2_ceil(E);
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const int base = blockIdx.x * kChunk;
-  for (int r = 0; r < kRounds; ++r) {
-    int f = base + r * kThreads + threadIdx.x;
+  int* next = smem + wv * E;
+  for (int e = lane; e < E; e += MOE_WAVE) next[e] = 0;   // (a wave's LDS accesses complete in program order)
+  const int base = blockIdx.x * kChunk + wv * kWaveSpan;
+  int my_id[kWaveRounds];
+#pragma unroll
+  for (int r = 0; r < kWaveRounds; ++r) {
+    const int f = base + r * MOE_WAVE + lane;
     int id = f < R ? ids[f] : -1;
     if (id >= E) id = -1;  // out-of-range ids are dropped rather than corrupting LDS
-    unsigned long long m = match_any(id, bits);
-    int rank = __popcll(m & ((1ull << lane) - 1ull));
-    int cnt = __popcll(m);
-    // waves take their turn in flat-index order so ranks stay stable
-    int pos = 0;
-    for (int turn = 0; turn < kWaves; ++turn) {
-      if (wv == turn && id >= 0) {
-        pos = next[id] + rank;  // every lane of a class reads before its leader bumps the counter
-      }
-      __syncthreads();
-      if (wv == turn && id >= 0 && rank == 0) next[id] += cnt;
-      __syncthreads();
+    my_id[r] = id;
+    const unsigned long long m = match_any(id, bits);
+    // the lowest lane of each match class adds the class size (one writer per counter and instruction)
+    if (id >= 0 && (m & ((1ull << lane) - 1ull)) == 0ull) next[id] += __popcll(m);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kThreads) {
+    int run = chunk_base[(size_t)blockIdx.x * E + e];
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int c = smem[w * E + e];
+      smem[w * E + e] = run;
+      run += c;
     }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < kWaveRounds; ++r) {
+    const int f = base + r * MOE_WAVE + lane;
+    const int id = my_id[r];
+    const unsigned long long m = match_any(id, bits);
+    const int rank = __popcll(m & ((1ull << lane) - 1ull));
     if (id >= 0) {
+      const int pos = next[id] + rank;   // every lane of a class reads before its leader bumps the counter
+      if (rank == 0) next[id] += __popcll(m);
       if (sort_order) sort_order[pos] = f;
       if (sorted_token_ids) sorted_token_ids[pos] = f / k;
       if (inv_perm) inv_perm[f] = pos;
@@ -294,10 +335,11 @@ int moe_permute_impl(const int32_t* idx, int M, int k, int E, int32_t* group_siz
   }
   int32_t* chunk_hist = (int32_t*)ws;
   hipLaunchKernelGGL(hist_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, chunk_hist);
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kMaxE), 0, s, chunk_hist, n_chunks, E, group_sizes, group_offsets,
-                     tiles);
+  const int cached = (long long)n_chunks * E <= kScanCacheInts;
+  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(kMaxE), cached ? (size_t)n_chunks * E * sizeof(int) : 0, s, chunk_hist,
+                     n_chunks, E, group_sizes, group_offsets, tiles, cached);
   if (R > 0 && (sorted_token_ids || sort_order || inv_perm))
-    hipLaunchKernelGGL(scatter_kernel, dim3(n_chunks), dim3(kThreads), E * sizeof(int), s, idx, R, E, k,
+    hipLaunchKernelGGL(scatter_kernel, dim3(n_chunks), dim3(kThreads), kWaves * E * sizeof(int), s, idx, R, E, k,
                        chunk_hist, sorted_token_ids, sort_order, inv_perm);
   return moe_check_hip(hipGetLastError(), "permute launch");
 }
