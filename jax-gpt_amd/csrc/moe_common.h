@@ -120,7 +120,8 @@ __device__ inline int moe_tile_first(int e, int E, int rows, int* lds_rows, int*
   // The two walks over all experts (the ranking; the tiles and cost in front of an expert) are shared out: with
   // epad = E rounded up to a power of two (at least a wavefront), the workgroup's threads form blockDim / epad parts,
   // thread (part, e2) walks the part's slice of the experts on behalf of expert e2, and the parts' sums meet in LDS
-  // (one thread per expert walking them all: 12 us of a 17 us launch for 128 experts).
+  // (against one thread per expert walking them all: 2 us less of a 17 us launch at 128 experts; most of such a
+  // launch is its start -- arguments, first instruction lines, first loads -- and not its arithmetic).
   int epad = 64;
   while (epad < E) epad <<= 1;
   const int parts = (int)blockDim.x / epad;          // >= 1: the caller has at least E threads, a power of two of them

@@ -170,6 +170,16 @@ template <int XF, int MODE = MODE_GATEUP> struct Cls {
   // what may still be in flight when a step starts that found every later copy issued: the activation stages and
   // weight stages of the steps after it
   static constexpr int IN_FLIGHT = (X_PRE - 1) * XS_OPS + (W_PRE - 1) * 8;
+  // The same count for a step rem = KB - 1 - kb steps from the item's end: the copies issued behind the last one that
+  // the step needs (its activation tile and scales, from X_PRE steps back), where a step that is r steps from the
+  // end issued activation copies if r >= X_PRE and weight copies if r >= W_PRE.
+  static constexpr int allowed(int rem) {
+    int n = 0;
+    if (X_FIRST && rem + X_PRE >= W_PRE) n += 8;   // the weight copies behind the needed ones in their own step
+    for (int r = rem + X_PRE - 1; r > rem; --r) n += (r >= X_PRE ? XS_OPS : 0) + (r >= W_PRE ? 8 : 0);
+    return n;
+  }
+  static_assert(allowed(W_PRE + X_PRE) == IN_FLIGHT, "the steady state of the rule is the count above");
   // copy operations issued after group g: spread over the first SPREAD groups of the step.  Rings of one depth must
   // have the step's copies out early (they land before the next barrier or hold it up); with the deeper weight ring
   // the weight copies have a step more, and an even spread over the whole step is best (all groups against the
@@ -346,9 +356,9 @@ __device__ __forceinline__ void item_body(const Item& item, uint8_t* lds, const 
         wait_vm<C::IN_FLIGHT>();
       } else {
         const int rem = KB - 1 - kb;        // the last steps: fewer and fewer copies are in flight
-        constexpr int one = (C::X_PRE > 1 ? C::XS_OPS : 0) + (C::W_PRE > 1 ? 8 : 0);   // the copies of one later step
-        if (rem >= 2) wait_vm<C::IN_FLIGHT>();
-        else if (rem == 1) wait_vm<one>();
+        static_assert(C::W_PRE <= 3, "steps that issue no weight copies are less than W_PRE from the end");
+        if (rem >= 2) wait_vm<C::allowed(2)>();
+        else if (rem == 1) wait_vm<C::allowed(1)>();
         else wait_vm<0>();
       }
       if (ROT > 0) wait_lgkm0();      // this wave's reads of stage kb - 1 are done before anyone overwrites it
