@@ -224,6 +224,31 @@ def test_grouped_gemms_vs_oracle(jg, E, D, I, sizes):
     assert np.mean(got_y != want_y) < 0.05           # same bf16 values except where 2^-16 crosses a rounding tie
 
 
+def test_gateup_full_height_tiles_same_bits_whatever_the_timing(jg):
+    """A 225-256 row gate/up tile refills a weight stage while the step that read it still computes; two waves agree
+    on the moment through a word in LDS.  The result must not depend on timing: the same expert's rows are computed
+    alone on an idle GPU and amid 63 others that keep every CU and the memory busy, the busy launch several times."""
+    import torch
+    _say("gateup timing independence")
+    E, D, I = 64, 2048, 256
+    sizes = [250 + (i % 7) for i in range(E)]
+    off, xq, sx, ex = _ragged_case(650, E, D, I, sizes)
+    dex = H.experts_to_cuda(ex)
+    dxq, dsx, doff = H.to_cuda(xq), H.to_cuda(sx), H.to_cuda(off)
+    hq0, sh0 = jg.gemm_gateup_swiglu(dxq, dsx, dex["gate_proj"], dex["up_proj"], doff)
+    for _ in range(5):
+        hq, sh = jg.gemm_gateup_swiglu(dxq, dsx, dex["gate_proj"], dex["up_proj"], doff)
+        assert torch.equal(hq.view(torch.uint8), hq0.view(torch.uint8)) and torch.equal(sh, sh0)
+    torch.cuda.synchronize()
+    for e in (0, 31, 63):
+        lo, hi = int(off[e]), int(off[e + 1])
+        one = {n: {"w": dex[n]["w"][e:e + 1], "scale_inv": dex[n]["scale_inv"][e:e + 1]} for n in ("gate_proj", "up_proj")}
+        hq1, sh1 = jg.gemm_gateup_swiglu(dxq[lo:hi].contiguous(), dsx[lo:hi].contiguous(), one["gate_proj"], one["up_proj"],
+                                         H.to_cuda(np.array([0, hi - lo], np.int32)))
+        assert torch.equal(hq1.view(torch.uint8), hq0[lo:hi].view(torch.uint8)), f"expert {e}: codes depend on the launch"
+        assert torch.equal(sh1, sh0[lo:hi]), f"expert {e}: scales depend on the launch"
+
+
 def test_grouped_gemm_row_ids_gather(jg):
     """row_ids reads activation rows through an index instead of a materialised x_sorted (moe.py:79)."""
     _say("gemm row_ids")
