@@ -193,9 +193,9 @@ def test_block_major_scales_give_the_same_bits(jg, E, D, I, sizes, gather):
     (2, 256, 256, [300, 150]),                    # two row tiles for one expert (near-equal cut), one 160-row tile for the other
     (2, 256, 256, [4200, 100]),                   # 17 row tiles: the column blocks are walked once per group of 8-9 row tiles
     (3, 1024, 256, [256, 0, 510]),                # 225-256 row tiles over 8 K steps: gate/up refills a weight stage inside the step that reads it
-    # the smallest experts form a pool that every XCD draws from behind its fixed share: the last round of 8 here ...
+    # the smallest experts form a pool that every XCD draws from behind its fixed share: the eight smallest of the ranking here ...
     (64, 256, 128, [500] * 48 + [3, 40, 17, 0, 1, 33, 25, 8, 12, 0, 31, 2, 64, 5, 9, 20]),
-    # ... and experts of two row tiles each in the pool here (one round of the three tail rounds fits the pool's limit)
+    # ... and experts of two row tiles each in the pool here (of the ranking's last three groups of eight, one fits the pool's limit)
     (200, 128, 128, [257 + (7 * i) % 44 for i in range(200)]),
 ])
 def test_grouped_gemms_vs_oracle(jg, E, D, I, sizes):
