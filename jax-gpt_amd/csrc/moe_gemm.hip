@@ -139,7 +139,7 @@ template <int XF, int MODE = MODE_GATEUP> struct Cls {
   // kb still computes, as if the ring were a stage deeper, in the same LDS.  The weight rows that wave (wi, 0) copies
   // are read by itself and by wave (wi, 1) alone, so the release is a word in LDS between those two (early_flag)
   // and no barrier.  Only the 256-row class of the gate/up GEMM, which has no room for a third stage: -4.5 % where
-  // every workgroup streams its own weight slab, -3 % where 8 row tiles share one, nothing on the mixed tile
+  // every workgroup streams its own weight slab, -3 % where 8 row tiles share one, -1 % on the mixed tile
   // heights of skewed routing; the down GEMM (16 K steps at the DeepSeek-V3 shape) gained 2 % in the first case and
   // lost 1 % in the second, and the classes with three weight stages cannot gain: their copies complete in issue
   // order behind the activation copies of the step before, which must have landed a step earlier.
