@@ -75,7 +75,8 @@ def test_sigmoid_scores_bit_exact(jg):
 # ---------------------------------------------------------------- permute
 
 @pytest.mark.parametrize("M,k,E,skew", [(256, 2, 8, False), (4096, 8, 128, False), (8192, 8, 256, False), (64, 8, 256, False),
-                                         (1, 1, 4, False), (3000, 4, 32, True), (513, 3, 1000, False)])
+                                         (1, 1, 4, False), (3000, 4, 32, True), (513, 3, 1000, False),
+                                         (6000, 6, 1000, False)])   # (chunks x experts beyond what the scan keeps in LDS)
 def test_permute_bit_exact(jg, M, k, E, skew):
     _say("permute", M, k, E, skew)
     rng = H.rng_for(300 + M)
